@@ -1,0 +1,35 @@
+"""Run-time settings of the engine (not read from config.json).
+
+The reference keeps the like in its builder (core/src/main/java/io/teknek/deliverance/
+model/AutoModelForCausaLm.java:106-134: working dtype, ``maxBatchSize`` 512, KV settings)
+and in ``AutoModelConfig`` (core/.../model/AutoModelConfig.java:20-33).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+DTYPE_NAMES = {"bfloat16": "bfloat16", "bf16": "bfloat16", "BF16": "bfloat16",
+               "float32": "float32", "fp32": "float32", "f32": "float32", "F32": "float32"}
+
+
+@dataclass
+class EngineConfig:
+    dtype: str = "bfloat16"            # "bfloat16" (serving kernels) or "float32" (true 32-bit)
+    page_size: int = 16                # tokens per KV page; a multiple of 16
+    max_cached_tokens: Optional[int] = None   # pool size in tokens; None: sized from free memory
+    max_num_seqs: int = 64             # live requests at a time
+    max_batch_tokens: int = 2048       # token budget of one step
+    max_chunk: int = 512               # largest prompt portion (the reference's maxBatchSize)
+    state_slots: Optional[int] = None  # slots for fixed-size per-request state; None: max_num_seqs
+    use_graphs: bool = True            # replay decode-only steps from captured HIP graphs
+    device: str = "cuda:0"
+
+    def __post_init__(self):
+        if self.dtype not in DTYPE_NAMES:
+            raise ValueError(f"dtype must be bfloat16 or float32, found {self.dtype!r}")
+        self.dtype = DTYPE_NAMES[self.dtype]
+        if self.page_size <= 0 or self.page_size % 16 != 0:
+            raise ValueError(f"page_size must be a positive multiple of 16, found {self.page_size}")
+        if self.max_num_seqs <= 0 or self.max_batch_tokens <= 0 or self.max_chunk <= 0:
+            raise ValueError("max_num_seqs, max_batch_tokens and max_chunk must be positive")

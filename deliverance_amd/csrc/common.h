@@ -1,0 +1,108 @@
+// Shared helpers of the gfx950 kernels: error reporting, dtype tags, bf16 conversion and
+// wave-level reductions.  Every entry point is `extern "C" int da_*(...)`: it validates its
+// arguments on the host, launches on the given stream and returns 0, or returns non-zero
+// after storing a message that `da_last_error()` hands out.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define DA_F32 0
+#define DA_BF16 1
+
+#define DA_ACT_NONE 0
+#define DA_ACT_GELU_TANH 1
+#define DA_ACT_GELU_ERF 2
+#define DA_ACT_RELU 3
+#define DA_ACT_SILU 4
+
+#define DA_WAVE 64
+
+extern "C" const char* da_last_error();
+void da_set_error(const char* fmt, ...);
+
+#define DA_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      da_set_error(__VA_ARGS__);         \
+      return 1;                          \
+    }                                    \
+  } while (0)
+
+#define DA_CHECK_LAUNCH(name)                                                      \
+  do {                                                                             \
+    hipError_t e_ = hipGetLastError();                                             \
+    if (e_ != hipSuccess) {                                                        \
+      da_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));          \
+      return 2;                                                                    \
+    }                                                                              \
+  } while (0)
+
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// Round to nearest even; NaN stays a quiet NaN (the reference's C side rounds the same
+// way: native/src/main/c/simd/vector_simd.c:23-41, except that it flushes subnormals).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct DTypeOf;
+template <> struct DTypeOf<float> { static const int value = DA_F32; };
+template <> struct DTypeOf<bf16_t> { static const int value = DA_BF16; };
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+__device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// Parameter vectors (norm gains, biases, tables) keep the dtype they were stored in; the
+// tag travels with the pointer.
+__device__ __forceinline__ float load_param(const void* p, int dtype, size_t i) {
+  return dtype == DA_BF16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+
+__device__ __forceinline__ void store_out(void* p, int dtype, size_t i, float v) {
+  if (dtype == DA_BF16) ((bf16_t*)p)[i] = f32_to_bf16(v);
+  else ((float*)p)[i] = v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = DA_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, DA_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = DA_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, DA_WAVE));
+  return v;
+}
+
+// The activations of a feed-forward, in 32-bit
+// (math/src/main/java/io/teknek/deliverance/math/ActivationFunction.java:13-21).
+__device__ __forceinline__ float apply_act(float x, int act) {
+  switch (act) {
+    case DA_ACT_GELU_TANH: {
+      const float c = 0.7978845608028654f;  // sqrt(2/pi)
+      return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+    }
+    case DA_ACT_GELU_ERF:
+      return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f));
+    case DA_ACT_RELU:
+      return fmaxf(x, 0.0f);
+    case DA_ACT_SILU:
+      return x / (1.0f + expf(-x));
+    default:
+      return x;
+  }
+}
+
+static inline int da_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

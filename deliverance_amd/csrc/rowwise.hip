@@ -1,0 +1,128 @@
+// Row-wise kernels: embedding (+ learned positions), LayerNorm (optionally on gathered
+// rows), and the write of new keys and values into the paged cache.
+#include "common.h"
+#include <stdarg.h>
+
+static thread_local char g_error[512] = "";
+
+extern "C" const char* da_last_error() { return g_error; }
+
+void da_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+// ------------------------------------------------------------------------------------------
+// x[n, :] = wte[token[n], :] + wpe[pos[n], :]      (32-bit sum, 32-bit result)
+// Reference: core/src/main/java/io/teknek/deliverance/model/gpt2/Gpt2Model.java:42-48
+// ------------------------------------------------------------------------------------------
+__global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                             const void* __restrict__ wte, int wte_dtype,
+                             const void* __restrict__ wpe, int wpe_dtype,
+                             float* __restrict__ x, int E) {
+  const int n = blockIdx.x;
+  const size_t trow = (size_t)tokens[n] * E;
+  const size_t prow = wpe ? (size_t)positions[n] * E : 0;
+  for (int i = threadIdx.x; i < E; i += blockDim.x) {
+    float v = load_param(wte, wte_dtype, trow + i);
+    if (wpe) v += load_param(wpe, wpe_dtype, prow + i);
+    x[(size_t)n * E + i] = v;
+  }
+}
+
+extern "C" int da_embed(const int* tokens, const int* positions, const void* wte, int wte_dtype,
+                        const void* wpe, int wpe_dtype, float* x, int N, int E, void* stream) {
+  DA_REQUIRE(N >= 0 && E > 0, "embed: bad sizes N=%d E=%d", N, E);
+  if (N == 0) return 0;
+  int threads = E >= 256 ? 256 : (E >= 128 ? 128 : 64);
+  hipLaunchKernelGGL(embed_kernel, dim3(N), dim3(threads), 0, (hipStream_t)stream, tokens, positions,
+                     wte, wte_dtype, wpe, wpe_dtype, x, E);
+  DA_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// LayerNorm over rows of 32-bit x; one wave per row; mean and centred variance in 32-bit.
+//   y = (x - mean) / sqrt(var + eps) * w + b        (var biased, eps inside the root)
+// Reference: core/src/main/java/io/teknek/deliverance/generator/LayerNorm.java:127-150
+// `rows` (optional) gathers: output row r is the norm of input row rows[r].
+// ------------------------------------------------------------------------------------------
+__global__ void layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                 const void* __restrict__ w, int w_dtype,
+                                 const void* __restrict__ b, int b_dtype, float eps,
+                                 void* __restrict__ y, int y_dtype, int R, int E) {
+  const int wave = threadIdx.x / DA_WAVE, lane = threadIdx.x % DA_WAVE;
+  const int r = blockIdx.x * (blockDim.x / DA_WAVE) + wave;
+  if (r >= R) return;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * E;
+  float s = 0.f;
+  for (int i = lane; i < E; i += DA_WAVE) s += xr[i];
+  const float mean = wave_sum(s) / (float)E;
+  float q = 0.f;
+  for (int i = lane; i < E; i += DA_WAVE) {
+    float d = xr[i] - mean;
+    q += d * d;
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(q) / (float)E + eps);
+  for (int i = lane; i < E; i += DA_WAVE) {
+    float v = (xr[i] - mean) * inv * load_param(w, w_dtype, i);
+    if (b) v += load_param(b, b_dtype, i);
+    store_out(y, y_dtype, (size_t)r * E + i, v);
+  }
+}
+
+extern "C" int da_layernorm(const float* x, const int* rows, const void* w, int w_dtype,
+                            const void* b, int b_dtype, float eps, void* y, int y_dtype, int R,
+                            int E, void* stream) {
+  DA_REQUIRE(R >= 0 && E > 0, "layernorm: bad sizes R=%d E=%d", R, E);
+  DA_REQUIRE(eps > 0.f, "layernorm: eps must be > 0");
+  if (R == 0) return 0;
+  const int waves = 4;
+  hipLaunchKernelGGL(layernorm_kernel, dim3(da_ceil_div(R, waves)), dim3(waves * DA_WAVE), 0,
+                     (hipStream_t)stream, x, rows, w, w_dtype, b, b_dtype, eps, y, y_dtype, R, E);
+  DA_CHECK_LAUNCH("layernorm");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Keys and values of the step's tokens go to their cache rows.
+// qkv: [N, ld] rows holding q | k | v; k starts at column k_off, v at v_off, each Hkv*D wide.
+// One cache slot (one layer's pages): [n_pages][2][Hkv][page][D]; slot_map[n] is
+// page_id * page + row, or -1 for a token whose keys are not kept.
+// Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:315-336
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
+                                T* __restrict__ cache, const int* __restrict__ slot_map, int Hkv,
+                                int D, int page) {
+  const int n = blockIdx.x;
+  const int slot = slot_map[n];
+  if (slot < 0) return;
+  const int pg = slot / page, row = slot % page;
+  const int W = Hkv * D;
+  const size_t page_elems = (size_t)2 * Hkv * page * D;
+  for (int i = threadIdx.x; i < 2 * W; i += blockDim.x) {
+    const int kv = i / W, c = i % W, h = c / D, d = c % D;
+    const T v = qkv[(size_t)n * ld + (kv ? v_off : k_off) + c];
+    cache[pg * page_elems + (((size_t)kv * Hkv + h) * page + row) * D + d] = v;
+  }
+}
+
+extern "C" int da_kv_write(const void* qkv, int dtype, int ld, int k_off, int v_off, void* cache,
+                           const int* slot_map, int N, int Hkv, int D, int page, void* stream) {
+  DA_REQUIRE(N >= 0 && Hkv > 0 && D > 0 && page > 0, "kv_write: bad sizes");
+  DA_REQUIRE(k_off >= 0 && v_off >= 0 && k_off + Hkv * D <= ld && v_off + Hkv * D <= ld,
+             "kv_write: k/v columns [%d,%d)+%d exceed the row length %d", k_off, v_off, Hkv * D, ld);
+  if (N == 0) return 0;
+  const int threads = 256;
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL(kv_write_kernel<bf16_t>, dim3(N), dim3(threads), 0, (hipStream_t)stream,
+                       (const bf16_t*)qkv, ld, k_off, v_off, (bf16_t*)cache, slot_map, Hkv, D, page);
+  else
+    hipLaunchKernelGGL(kv_write_kernel<float>, dim3(N), dim3(threads), 0, (hipStream_t)stream,
+                       (const float*)qkv, ld, k_off, v_off, (float*)cache, slot_map, Hkv, D, page);
+  DA_CHECK_LAUNCH("kv_write");
+  return 0;
+}

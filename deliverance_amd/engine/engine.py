@@ -1,0 +1,201 @@
+"""The engine as a user sees it: load a model folder, generate tokens for prompts.
+
+In the reference's manner (README.md:84-107; core/src/test/java/io/teknek/deliverance/
+integration/Gpt2IT.java:25-36)::
+
+    model = AutoModelForCausalLM.from_pretrained(folder, dtype="bfloat16")
+    response = model.generate(prompt_ids, GeneratorParameters().with_temperature(0.0)
+                              .with_ntokens(500).with_max_tokens(150), on_token)
+
+``Response`` carries what the reference's does for an engine that works on token ids
+(core/.../generator/Response.java:10-22): generated tokens, finish reason, prompt tokens and
+the three timings.  Several prompts may be given at once; they are batched continuously.
+"""
+from __future__ import annotations
+
+import struct
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..kernels import ops
+from ..models.causal_lm import CausalLM, load_model
+from ..parts.base import KVNeed
+from ..sampling.params import GeneratorParameters
+from ..sampling.sampler import RECORD_WORDS, device_record
+from .device_cache import DeviceCache
+from .scheduler import Request, Scheduled, Scheduler
+from .step import StepEntry, StepRunner
+
+_TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class Response:
+    generated_tokens: List[int]
+    finish_reason: str                  # "length" | "stop" | "error" | "cancelled"
+    prompt_tokens: int
+    time_to_first_token_ms: float = 0.0
+    avg_time_per_token_ms: float = 0.0
+    total_time_ms: float = 0.0
+    top_logprobs: List[list] = field(default_factory=list)
+    error: Optional[str] = None
+    preemptions: int = 0
+
+
+class CausalLanguageModel:
+    """A loaded model with its cache, step function and scheduler on one GPU."""
+
+    def __init__(self, model: CausalLM, engine_config: EngineConfig):
+        if not torch.cuda.is_available():
+            raise RuntimeError("deliverance_amd runs on a GPU only; no device is visible")
+        self.model = model
+        self.config = model.config
+        self.engine_config = engine_config
+        needs = model.cache_needs()
+        tokens = engine_config.max_cached_tokens
+        if tokens is None:
+            free, _ = torch.cuda.mem_get_info(model.device)
+            tokens = DeviceCache.tokens_for_budget(needs, model.dtype, int(free * 0.5))
+            tokens = min(tokens, engine_config.max_num_seqs * model.config.max_positions)
+            tokens = max(tokens, engine_config.page_size)
+        n_slots = engine_config.state_slots if engine_config.state_slots is not None else engine_config.max_num_seqs
+        self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots)
+        self.runner = StepRunner(model, self.cache)
+        self.scheduler = Scheduler(self.cache.manager, model.config.max_positions, model.config.eos_token_ids,
+                                   engine_config.max_num_seqs, engine_config.max_batch_tokens,
+                                   engine_config.max_chunk, on_open=self.cache.reset_state)
+        self._next_id = 0
+        self._callbacks: Dict[Hashable, Callable] = {}
+        self._sampled_dev = torch.empty(max(engine_config.max_num_seqs, 64), dtype=torch.int32, device=model.device)
+
+    # ---- lower level: requests and steps -------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], params: Optional[GeneratorParameters] = None,
+                    rid: Optional[Hashable] = None, on_token: Optional[Callable] = None) -> Hashable:
+        if rid is None:
+            rid = self._next_id
+            self._next_id += 1
+        for t in prompt:
+            if not (0 <= int(t) < self.config.vocab_size):
+                raise ValueError(f"token id {t} is outside the vocabulary of {self.config.vocab_size}")
+        self.scheduler.add(rid, [int(t) for t in prompt], params or GeneratorParameters())
+        if on_token is not None:
+            self._callbacks[rid] = on_token
+        return rid
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def step(self) -> List[Request]:
+        """One scheduler decision, one model step, one sampling call.  Returns the requests
+        that finished in this step."""
+        before = len(self.scheduler.finished)
+        batch: List[Scheduled] = self.scheduler.schedule()
+        failed = self.scheduler.finished[before:]
+        if not batch:
+            return list(failed)
+        V = self.config.vocab_size
+        entries = []
+        records: List[int] = []
+        samplers: List[Scheduled] = []
+        for s in batch:
+            req = s.request
+            entries.append(StepEntry(req.rid, req.tokens_from(s.start, s.n), [s.n - 1] if s.samples else []))
+            if s.samples:
+                records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))
+                samplers.append(s)
+        logits, ctx = self.runner.run(entries, reserved=True, extra_words=records or None)
+        sampled: Dict[Hashable, int] = {}
+        if samplers:
+            R = len(samplers)
+            if self._sampled_dev.numel() < R:
+                self._sampled_dev = torch.empty(2 * R, dtype=torch.int32, device=self.model.device)
+            out = self._sampled_dev[:R]
+            ops.sample(logits, ctx.extra, out)
+            want_lp = [s for s in samplers if s.request.params.log_probs and s.request.params.top_log_probs > 0]
+            lp = None
+            if want_lp:
+                n = max(s.request.params.top_log_probs for s in want_lp)
+                idx = torch.empty((R, n), dtype=torch.int32, device=self.model.device)
+                val = torch.empty((R, n), dtype=torch.float32, device=self.model.device)
+                ops.top_logprobs(logits, ctx.extra, n, idx, val)
+                lp = (idx.cpu(), val.cpu())
+            host = out.cpu()                                   # the step's one synchronisation
+            for i, s in enumerate(samplers):
+                sampled[s.request.rid] = int(host[i])
+                p = s.request.params
+                if lp is not None and p.log_probs and p.top_log_probs > 0:
+                    k = p.top_log_probs
+                    s.request.top_logprobs.append(list(zip(lp[0][i, :k].tolist(), lp[1][i, :k].tolist())))
+        done = self.scheduler.complete(batch, sampled)
+        now = time.perf_counter()
+        for s in samplers:
+            cb = self._callbacks.get(s.request.rid)
+            if cb is not None:
+                cb(sampled[s.request.rid], s.request.rid, (now - s.request.t_arrival) * 1e3)
+        for r in done:
+            self._callbacks.pop(r.rid, None)
+        return list(failed) + done
+
+    # ---- the entry point ---------------------------------------------------------------------
+    def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],
+                 params: Union[None, GeneratorParameters, Sequence[GeneratorParameters]] = None,
+                 on_token: Optional[Callable] = None) -> Union[Response, List[Response]]:
+        """Generate for one prompt (a list of token ids) or several (a list of lists).
+        ``on_token(token, request_index, ms_since_arrival)`` is called for every new token, as
+        the reference's ``GenerateEvent.emit`` is (core/.../model/GenerateEvent.java:3-12)."""
+        single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
+        plist = [prompts] if single else list(prompts)
+        if params is None or isinstance(params, GeneratorParameters):
+            pl = [params or GeneratorParameters()] * len(plist)
+        else:
+            pl = list(params)
+            if len(pl) != len(plist):
+                raise ValueError("one GeneratorParameters per prompt is needed")
+        rids = []
+        for i, (pr, pa) in enumerate(zip(plist, pl)):
+            cb = None if on_token is None else (lambda tok, rid, ms, i=i: on_token(tok, i, ms))
+            rids.append(self.add_request(pr, pa, on_token=cb))
+        mine = set(rids)
+        got: Dict[Hashable, Request] = {}
+        while len(got) < len(rids):
+            if not self.has_work():
+                raise RuntimeError("the scheduler ran out of work before every request finished")
+            for r in self.step():
+                if r.rid in mine:
+                    got[r.rid] = r
+        out = [self._response(got[r]) for r in rids]
+        for r in rids:
+            self.scheduler.finished.remove(got[r])
+        return out[0] if single else out
+
+    @staticmethod
+    def _response(r: Request) -> Response:
+        """Timing as the reference computes it (core/.../model/GenerationEngine.java:249-268)."""
+        end = r.t_finish or time.perf_counter()
+        total = (end - r.t_arrival) * 1e3
+        ttft = ((r.t_first_token or end) - r.t_arrival) * 1e3
+        n = len(r.output)
+        return Response(list(r.output), r.finish_reason or "error", len(r.prompt), ttft,
+                        total / n if n else 0.0, total, list(r.top_logprobs), r.error, r.n_preempted)
+
+    def stats(self) -> dict:
+        d = dict(self.scheduler.counters)
+        d.update(self.cache.manager.stats())
+        return d
+
+
+class AutoModelForCausalLM:
+    """``from_pretrained`` reads config.json, picks the model by its architecture name and loads
+    the tensors by name (the reference: core/.../model/AutoModelForCausaLm.java:92-103,457-520)."""
+
+    @staticmethod
+    def from_pretrained(folder: str, dtype: str = "bfloat16", engine_config: Optional[EngineConfig] = None,
+                        **kwargs) -> CausalLanguageModel:
+        import deliverance_amd.models  # noqa: F401  (registers the architectures)
+        ec = engine_config or EngineConfig(dtype=dtype, **kwargs)
+        model = load_model(folder, _TORCH_DTYPE[ec.dtype], ec.device)
+        return CausalLanguageModel(model, ec)

@@ -1,0 +1,216 @@
+"""Python faces of the HIP kernels.
+
+Each function checks on the host that the operands have the shapes, dtypes and layout the
+kernel and its grid assume, then launches on torch's current stream.  Nothing here falls
+back to a library or to the CPU: a missing kernel library is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, found {t.dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise KernelError(build.load().da_last_error().decode())
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU")
+
+
+def _rows_2d(t: torch.Tensor, name: str):
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with a contiguous last dimension")
+
+
+# ------------------------------------------------------------------------------- embedding
+def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
+          wpe: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out[n] = wte[tokens[n]] + wpe[positions[n]] in 32-bit."""
+    _dev(tokens, positions, wte, wpe, out)
+    N, E = out.shape
+    _need(tokens.dtype == torch.int32 and positions.dtype == torch.int32, "embed: ids must be int32")
+    _need(tokens.numel() >= N and positions.numel() >= N, "embed: fewer ids than rows")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+    _need(wte.is_contiguous() and wte.shape[1] == E, "embed: token table width differs from out")
+    if wpe is not None:
+        _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: position table width differs from out")
+    _check(build.load().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
+                                 _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------- norms
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+              out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """LayerNorm of 32-bit rows; with ``rows`` the output row r is the norm of x[rows[r]]."""
+    _dev(x, weight, bias, out, rows)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2, "layernorm: x must be contiguous float32 [N, E]")
+    E = x.shape[1]
+    R = out.shape[0]
+    _need(out.is_contiguous() and out.shape[1] == E, "layernorm: out must be contiguous [R, E]")
+    _need(weight.numel() == E and (bias is None or bias.numel() == E), "layernorm: parameter length differs from E")
+    if rows is None:
+        _need(R <= x.shape[0], "layernorm: more output rows than input rows")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= R, "layernorm: rows must be int32 with R entries")
+    _check(build.load().da_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), _ptr(bias),
+                                     _dt(bias) if bias is not None else 0, ctypes.c_float(eps), _ptr(out),
+                                     _dt(out), R, E, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------- products
+def linear_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+               act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
+    """out (+)= act(a @ w.T + bias) with the plain tiled kernel; w is [N, K]."""
+    _dev(a, w, bias, out)
+    _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    _need(out.shape[0] == M and out.shape[1] == N, f"linear: out is {list(out.shape)}, expected [{M},{N}]")
+    _need(a.dtype == w.dtype, "linear: a and w must share a dtype")
+    _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
+    _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
+    _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
+    _check(build.load().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
+                                    _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
+                                    _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------- cache write
+def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.Tensor,
+             slot_map: torch.Tensor, n_kv_heads: int, head_dim: int) -> None:
+    """Rows of k and v (columns k_off.., v_off.. of qkv) go to cache rows ``slot_map``.
+    cache_slot: [n_pages, 2, Hkv, page, D]."""
+    _dev(qkv, cache_slot, slot_map)
+    _rows_2d(qkv, "qkv")
+    N = qkv.shape[0]
+    _need(cache_slot.dim() == 5 and cache_slot.is_contiguous(), "kv_write: cache slot must be contiguous [pages,2,Hkv,page,D]")
+    P, two, Hkv, page, D = cache_slot.shape
+    _need(two == 2 and Hkv == n_kv_heads and D == head_dim, "kv_write: cache slot shape differs from the heads")
+    _need(cache_slot.dtype == qkv.dtype, "kv_write: cache and activations differ in dtype")
+    _need(slot_map.dtype == torch.int32 and slot_map.numel() >= N, "kv_write: slot_map must be int32 [N]")
+    _check(build.load().da_kv_write(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot),
+                                    _ptr(slot_map), N, Hkv, D, page, _stream()))
+
+
+# ------------------------------------------------------------------------------- attention
+def attention_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
+                  seq_of_token: torch.Tensor, positions: torch.Tensor, n_heads: int, scale: float,
+                  window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+    """Plain paged attention for any rows.  q: [N, >= Hq*D] view (row stride free)."""
+    _dev(q, cache_slot, block_table, seq_of_token, positions, out)
+    _rows_2d(q, "q"); _rows_2d(out, "out")
+    N = q.shape[0]
+    P, two, Hkv, page, D = cache_slot.shape
+    _need(cache_slot.is_contiguous() and two == 2, "attention: cache slot must be contiguous [pages,2,Hkv,page,D]")
+    _need(q.shape[1] == n_heads * D and out.shape[1] == n_heads * D and out.shape[0] == N,
+          "attention: q/out must be [N, Hq*D]")
+    _need(q.dtype == cache_slot.dtype == out.dtype, "attention: q, cache and out must share a dtype")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "attention: block_table must be contiguous int32 [S, max_blocks]")
+    _need(seq_of_token.dtype == torch.int32 and positions.dtype == torch.int32, "attention: ids must be int32")
+    _need(seq_of_token.numel() >= N and positions.numel() >= N, "attention: fewer ids than rows")
+    _check(build.load().da_attn_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table),
+                                    block_table.shape[1], _ptr(seq_of_token), _ptr(positions), N, n_heads, Hkv,
+                                    D, page, ctypes.c_float(scale), int(window or 0), _ptr(out), out.stride(0),
+                                    _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------- sampling
+SAMPLE_ROW_FLOATS = 8     # one SampleRow record is 8 four-byte fields
+
+
+def sample(logits: torch.Tensor, params: torch.Tensor, out_tokens: torch.Tensor) -> torch.Tensor:
+    """params: int32/float32-punned [R, 8] records (see sampling.device_rows)."""
+    _dev(logits, params, out_tokens)
+    _rows_2d(logits, "logits")
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "sample: logits must be float32")
+    _need(params.is_contiguous() and params.numel() >= R * SAMPLE_ROW_FLOATS and params.element_size() == 4,
+          "sample: params must hold R records of 8 four-byte fields")
+    _need(out_tokens.dtype == torch.int32 and out_tokens.numel() >= R, "sample: out must be int32 [R]")
+    _check(build.load().da_sample(_ptr(logits), logits.stride(0), R, V, _ptr(params), _ptr(out_tokens), _stream()))
+    return out_tokens
+
+
+def top_logprobs(logits: torch.Tensor, params: torch.Tensor, n: int, out_idx: torch.Tensor,
+                 out_lp: torch.Tensor) -> None:
+    _dev(logits, params, out_idx, out_lp)
+    _rows_2d(logits, "logits")
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "top_logprobs: logits must be float32")
+    _need(0 < n <= V, "top_logprobs: n must be in [1, V]")
+    _need(out_idx.dtype == torch.int32 and out_idx.numel() >= R * n and out_idx.is_contiguous(), "top_logprobs: out_idx")
+    _need(out_lp.dtype == torch.float32 and out_lp.numel() >= R * n and out_lp.is_contiguous(), "top_logprobs: out_lp")
+    _check(build.load().da_top_logprobs(_ptr(logits), logits.stride(0), R, V, _ptr(params), n, _ptr(out_idx),
+                                        _ptr(out_lp), _stream()))
+
+
+# ------------------------------------------------------------------------------- dispatch
+# "tuned": MFMA products and the prefill/decode attention kernels in bfloat16;
+# "reference": the plain kernels everywhere (for A/B checks).  32-bit always runs the plain
+# kernels: they are its product path.
+_MODE = "tuned"
+
+
+def set_kernel_mode(mode: str) -> None:
+    global _MODE
+    if mode not in ("tuned", "reference"):
+        raise ValueError("kernel mode must be 'tuned' or 'reference'")
+    _MODE = mode
+
+
+def kernel_mode() -> str:
+    return _MODE
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+           act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
+    """out (+)= act(a @ w.T + bias); picks the kernel by dtype and mode."""
+    return linear_ref(a, w, bias, out, act, accumulate)
+
+
+def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int,
+                    scale: float, window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+    """Attention of every row of the step over its sequence's pages."""
+    return attention_ref(q, cache_slot, ctx.block_tables[group], ctx.seq_of_token, ctx.positions,
+                         n_heads, scale, window, out)

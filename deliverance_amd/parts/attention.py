@@ -1,0 +1,62 @@
+"""Causal self-attention over the paged cache, as a mixer.
+
+Fused projection to q | k | v (+ bias), optional position encoding of q and k, write of the
+new k and v rows into the cache slot, attention of every row over its sequence's pages, and
+the output projection (+ bias) added into the residual stream.
+Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:226-420
+(projections :266-291, cache write :315-336, scores/softmax/weighted sum :458-532, output
+projection :385-408); the residual add is TransformerBlock.java:176.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import (KVNeed, Mixer, StepContext, build_position, register_mixer, to_matrix, to_vector)
+
+
+class CausalSelfAttention(Mixer):
+    def __init__(self, spec, params, dtype, device):
+        self.spec = spec
+        self.n_heads, self.n_kv_heads, self.head_dim = spec.n_heads, spec.n_kv_heads, spec.head_dim
+        if self.n_heads % self.n_kv_heads != 0:
+            raise ValueError(f"{self.n_heads} query heads are not a multiple of {self.n_kv_heads} key heads")
+        if self.head_dim % 16 != 0 or self.head_dim > 256:
+            raise ValueError(f"head size {self.head_dim} is not a multiple of 16 up to 256")
+        self.q_cols = self.n_heads * self.head_dim
+        self.kv_cols = self.n_kv_heads * self.head_dim
+        self.qkv_cols = self.q_cols + 2 * self.kv_cols
+        self.scale = float(spec.scale)
+        self.window = spec.window
+        self.qkv_weight = to_matrix(params["qkv_weight"], dtype, device)
+        self.out_weight = to_matrix(params["out_weight"], dtype, device)
+        self.qkv_bias = to_vector(params.get("qkv_bias"), dtype, device) if spec.qkv_bias else None
+        self.out_bias = to_vector(params.get("out_bias"), dtype, device) if spec.out_bias else None
+        if tuple(self.qkv_weight.shape) != (self.qkv_cols, spec.width):
+            raise ValueError(f"qkv weight is {list(self.qkv_weight.shape)}, expected {[self.qkv_cols, spec.width]}")
+        if tuple(self.out_weight.shape) != (spec.width, self.q_cols):
+            raise ValueError(f"output weight is {list(self.out_weight.shape)}, expected {[spec.width, self.q_cols]}")
+        self.position = None
+        if spec.position is not None and spec.position.kind != "none":
+            self.position = build_position(spec.position, params.get("position", {}), dtype, device)
+
+    def cache_need(self):
+        return KVNeed(self.n_kv_heads, self.head_dim, self.window)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
+        N = h.shape[0]
+        qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
+        ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
+        if self.position is not None:
+            self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
+        slot = ctx.cache.kv[call.cache]
+        group = ctx.group_of(call.cache)
+        if call.write:
+            ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
+                         self.n_kv_heads, self.head_dim)
+        o = ctx.buf("attn_out", N, self.q_cols, ctx.dtype)
+        ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
+        ops.linear(o, self.out_weight, self.out_bias, x, accumulate=True)
+
+
+register_mixer("attention", CausalSelfAttention)

@@ -1,0 +1,86 @@
+"""Trace replay: feed given token ids through a model step by step and write logits.
+
+It samples nothing and decides nothing: every step of the trace becomes one call of the
+engine's own step function, on the engine's own model, cache manager and kernels.  The
+nearest thing in the reference is a test helper that compares cached decoding with a cold
+replay (core/src/test/java/io/teknek/deliverance/model/hf/HfGenerationTesterMixinPort.java:16-36).
+
+Input, one JSON object a line::
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+For a step in which something is wanted, ``<out>/<step>.f32`` holds the logits at the wanted
+places, in the order of the entries and of ``want``, as little-endian float32 [wanted, vocab].
+After every step a line ``done <step>`` is printed and flushed.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for the <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--page-size", type=int, default=16)
+    args = ap.parse_args(argv)
+
+    def say(msg):
+        print(f"[trace_run] {msg}", file=sys.stderr, flush=True)
+
+    say("importing torch")
+    import torch
+    from .kernels import build
+    if build.library_path() is None:
+        say("compiling the HIP kernels (first call)")
+    build.load()
+    if not torch.cuda.is_available():
+        say("no GPU is visible; trace_run drives the GPU engine and has no other path")
+        return 3
+    from . import models  # noqa: F401
+    from .engine.device_cache import DeviceCache
+    from .engine.step import StepEntry, StepRunner
+    from .models.causal_lm import load_model
+
+    if args.page_size <= 0 or 64 % args.page_size != 0:
+        say("--page-size must divide 64")
+        return 2
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    say(f"loading {args.model} as {args.dtype}")
+    model = load_model(args.model, dtype, "cuda:0")
+    # A request's count is rounded up to a multiple of 64, so max_tokens / page_size pages hold
+    # every live request whatever its length.
+    cache = DeviceCache(model.cache_needs(), dtype, "cuda:0", args.page_size, max(args.max_tokens, 64),
+                        n_state_slots=8)
+    runner = StepRunner(model, cache)
+    os.makedirs(args.out, exist_ok=True)
+    say("ready")
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        step = rec["step"]
+        entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
+        if entries:
+            logits, _ = runner.run(entries)
+            if logits.shape[0]:
+                logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4").tofile(
+                    os.path.join(args.out, f"{step}.f32"))
+            else:
+                torch.cuda.synchronize()
+        for rid in rec.get("end", []):
+            cache.manager.close(rid)
+        print(f"done {step}", flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
