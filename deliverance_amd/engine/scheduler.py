@@ -228,6 +228,7 @@ class Scheduler:
             req = s.request
             if req.state != RUNNING:
                 continue
+            self.cache.commit(req.rid)
             req.n_computed = s.start + s.n
             if not s.samples:
                 continue

@@ -181,6 +181,7 @@ class StepRunner:
         self.last_ctx = ctx
 
         logits = self.model.forward(ctx, view("want") if R else None, R)
-        for e in entries:
-            mgr.commit(e.rid)
+        if not reserved:                 # who reserves commits: the scheduler does it for its batches
+            for e in entries:
+                mgr.commit(e.rid)
         return logits, ctx

@@ -21,6 +21,43 @@ import os
 import sys
 
 
+class TraceSession:
+    """The engine's model, cache and step function, driven one trace step at a time."""
+
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0"):
+        import torch
+        from . import models  # noqa: F401  (registers the architectures)
+        from .engine.device_cache import DeviceCache
+        from .engine.step import StepRunner
+        from .models.causal_lm import load_model
+        if page_size <= 0 or 64 % page_size != 0:
+            raise ValueError("page size must divide 64")
+        tdtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
+        self.model = load_model(model_dir, tdtype, device)
+        # A request's count is rounded up to a multiple of 64, so max_tokens / page_size pages
+        # hold every live request whatever its length.
+        self.cache = DeviceCache(self.model.cache_needs(), tdtype, device, page_size, max(max_tokens, 64),
+                                 n_state_slots=8)
+        self.runner = StepRunner(self.model, self.cache)
+
+    def run_step(self, rec: dict):
+        """One line of the trace.  Returns the wanted logits as a float32 array [wanted, vocab],
+        or None when nothing was wanted."""
+        import torch
+        from .engine.step import StepEntry
+        entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
+        out = None
+        if entries:
+            logits, _ = self.runner.run(entries)
+            if logits.shape[0]:
+                out = logits.detach().to("cpu", torch.float32).contiguous().numpy()
+            else:
+                torch.cuda.synchronize()
+        for rid in rec.get("end", []):
+            self.cache.manager.close(rid)
+        return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__,
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -29,7 +66,7 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder for the <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
-    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page; divides 64")
     args = ap.parse_args(argv)
 
     def say(msg):
@@ -44,22 +81,8 @@ def main(argv=None) -> int:
     if not torch.cuda.is_available():
         say("no GPU is visible; trace_run drives the GPU engine and has no other path")
         return 3
-    from . import models  # noqa: F401
-    from .engine.device_cache import DeviceCache
-    from .engine.step import StepEntry, StepRunner
-    from .models.causal_lm import load_model
-
-    if args.page_size <= 0 or 64 % args.page_size != 0:
-        say("--page-size must divide 64")
-        return 2
-    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     say(f"loading {args.model} as {args.dtype}")
-    model = load_model(args.model, dtype, "cuda:0")
-    # A request's count is rounded up to a multiple of 64, so max_tokens / page_size pages hold
-    # every live request whatever its length.
-    cache = DeviceCache(model.cache_needs(), dtype, "cuda:0", args.page_size, max(args.max_tokens, 64),
-                        n_state_slots=8)
-    runner = StepRunner(model, cache)
+    session = TraceSession(args.model, args.dtype, args.max_tokens, args.page_size)
     os.makedirs(args.out, exist_ok=True)
     say("ready")
     for line in sys.stdin:
@@ -67,18 +90,10 @@ def main(argv=None) -> int:
         if not line:
             continue
         rec = json.loads(line)
-        step = rec["step"]
-        entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
-        if entries:
-            logits, _ = runner.run(entries)
-            if logits.shape[0]:
-                logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4").tofile(
-                    os.path.join(args.out, f"{step}.f32"))
-            else:
-                torch.cuda.synchronize()
-        for rid in rec.get("end", []):
-            cache.manager.close(rid)
-        print(f"done {step}", flush=True)
+        logits = session.run_step(rec)
+        if logits is not None:
+            logits.astype("<f4").tofile(os.path.join(args.out, f"{rec['step']}.f32"))
+        print(f"done {rec['step']}", flush=True)
     return 0
 
 

@@ -99,20 +99,29 @@ def softmax_rows(s):
     return e / e.sum(axis=-1, keepdims=True)
 
 
-def causal_attention(q, k, v, n_head, scale, window=None):
+def causal_attention(q, k, v, n_head, scale, window=None, n_kv_head=None, past=0):
     """Per head h (columns h*D .. h*D+D-1, core/.../generator/CausalSelfAttention.java:478-479):
     scores q_t . k_j * scale for j <= t only (CausalSelfAttention.java:481-491,512-527),
-    softmax, weighted sum of v.  ``window`` w keeps only the last w keys (t-w < j <= t)."""
-    T, E = q.shape
-    D = E // n_head
+    softmax, weighted sum of v.  ``window`` w keeps only the last w keys (t-w < j <= t).
+    With fewer key heads, query head h reads key head h // (n_head / n_kv_head)
+    (tensor/src/test/java/io/teknek/deliverance/tensor/operations/
+    TensorOperationsDecodePagedAttentionTest.java:49-57).  ``past``: q holds the last
+    len(q) positions of a sequence whose keys are all in k, v."""
+    T = q.shape[0]
+    D = q.shape[1] // n_head
+    n_kv_head = n_kv_head or n_head
+    group = n_head // n_kv_head
     out = np.zeros_like(q)
     for h in range(n_head):
-        qh, kh, vh = (a[:, h * D:(h + 1) * D] for a in (q, k, v))
+        g = h // group
+        qh = q[:, h * D:(h + 1) * D]
+        kh, vh = k[:, g * D:(g + 1) * D], v[:, g * D:(g + 1) * D]
         for t in range(T):
-            lo = 0 if window is None else max(0, t - window + 1)
-            s = (kh[lo:t + 1] @ qh[t]) * scale
+            p = past + t
+            lo = 0 if window is None else max(0, p - window + 1)
+            s = (kh[lo:p + 1] @ qh[t]) * scale
             w = softmax_rows(s[None, :])[0]
-            out[t, h * D:(h + 1) * D] = w @ vh[lo:t + 1]
+            out[t, h * D:(h + 1) * D] = w @ vh[lo:p + 1]
     return out
 
 
