@@ -1,0 +1,171 @@
+// Paged attention for decode rows in bfloat16: one query row per sequence.
+//
+// One workgroup of 4 wavefronts per (sequence, query head).  The keys lo..p of the sequence
+// are walked in aligned chunks of 64; wavefront v takes chunks v, v+4, ...
+//   scores : CPR lanes share a key, each holding a 16-byte piece of the key row and the matching
+//            piece of q in registers; their partial dot products are added by lane exchange.
+//            One load instruction so covers 64 / CPR whole key rows that lie next to each other.
+//   softmax: every lane ends up with one key's score; running maximum and sum per wavefront
+//            (the recurrence of native/src/main/resources/decode_paged_attention_f32.wgsl:31-65).
+//   values : values are stored dimension-major, so lane d reads 8 consecutive keys of its own
+//            dimension in 16 bytes and keeps one accumulator; no exchange between lanes.
+// The four wavefronts' partial results are merged in LDS in a fixed order.  Every sum's order
+// depends on p and lo only, never on the batch.
+//
+// Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:504-532;
+// tensor/src/main/java/io/teknek/deliverance/tensor/operations/TensorOperations.java:240-272.
+#include "common.h"
+
+#define DEC_WAVES 4
+#define DEC_MAX_D 256
+#define DEC_DPL (DEC_MAX_D / DA_WAVE)   // value dimensions per lane at most
+
+// CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
+template <int CPR>
+__global__ void __launch_bounds__(DEC_WAVES * DA_WAVE)
+attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
+                   const int* __restrict__ block_table, int max_blocks,
+                   const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
+                   int window, bf16_t* __restrict__ out, int out_ld) {
+  constexpr int G = DA_WAVE / CPR;            // keys scored side by side
+  __shared__ __attribute__((aligned(16))) float ps[DEC_WAVES][DA_WAVE];
+  __shared__ float part_acc[DEC_WAVES][DEC_MAX_D];
+  __shared__ float part_m[DEC_WAVES], part_l[DEC_WAVES];
+
+  const int s = blockIdx.x / Hq, h = blockIdx.x % Hq;
+  const int hk = h / (Hq / Hkv);
+  const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
+  const int p = seq_lens[s] - 1;                      // the row's position; it sees keys lo..p
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int* bt = block_table + (size_t)s * max_blocks;
+
+  const int piece = lane % CPR, sub = lane / CPR;
+  const bool piece_ok = piece * 8 < D;
+  float qf[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    qf[e] = piece_ok ? bf16_to_f32(q[(size_t)s * q_ld + h * D + piece * 8 + e]) * scale : 0.f;
+
+  float acc[DEC_DPL];
+#pragma unroll
+  for (int i = 0; i < DEC_DPL; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  for (int c0 = (lo / DA_WAVE) * DA_WAVE + wave * DA_WAVE; c0 <= p; c0 += DEC_WAVES * DA_WAVE) {
+    // ---- scores: iteration i handles keys c0 + i*G + sub
+    float mine = -INFINITY;      // one key's score per lane, once the loop is done
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) {
+      const int key = c0 + i * G + sub;
+      const bool valid = key >= lo && key <= p;
+      float dot = 0.f;
+      if (valid && piece_ok) {
+        const bf16_t* kr = cache + cache_k_row(bt[key / page], hk, key % page, Hkv, page, D) + piece * 8;
+        const uint4 kv = *(const uint4*)kr;
+        const uint32_t u[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dot = fmaf(qf[2 * e], __uint_as_float(u[e] << 16), dot);
+          dot = fmaf(qf[2 * e + 1], __uint_as_float(u[e] & 0xffff0000u), dot);
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < CPR; o <<= 1) dot += __shfl_xor(dot, o, DA_WAVE);
+      // all CPR lanes of the group now hold the score; the lane whose piece number is i keeps it
+      if (piece == i) mine = valid ? dot : -INFINITY;
+    }
+    const int kidx = piece * G + sub;                 // which key of the chunk this lane kept
+    const int key = c0 + kidx;
+    const bool valid = key >= lo && key <= p;
+    const float m_new = fmaxf(m, wave_max(mine));
+    const float e = valid ? expf(mine - m_new) : 0.f;
+    const float alpha = expf(m - m_new);
+    l = l * alpha + wave_sum(e);
+    m = m_new;
+    ps[wave][kidx] = e;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // ---- values: lane owns dimensions lane, lane + 64, ...
+    const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
+    const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
+#pragma unroll
+    for (int i = 0; i < DEC_DPL; ++i) {
+      const int d = lane + i * DA_WAVE;
+      if (d >= D) break;
+      float a = acc[i] * alpha;
+      for (int g0 = (first / 8) * 8; g0 <= last; g0 += 8) {   // groups of 8 keys, never across a page
+        const bf16_t* vr = cache + cache_v_base(bt[g0 / page], hk, Hkv, page, D) + (long long)d * page + g0 % page;
+        const uint4 vv = *(const uint4*)vr;
+        const uint32_t u[4] = {vv.x, vv.y, vv.z, vv.w};
+        const float4 w0 = *(const float4*)&ps[wave][g0 - c0];
+        const float4 w1 = *(const float4*)&ps[wave][g0 - c0 + 4];
+        const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          // rows outside first..last were never written (or belong to someone else): keep them out
+          const float v0 = (g0 + 2 * e2 >= first && g0 + 2 * e2 <= last) ? __uint_as_float(u[e2] << 16) : 0.f;
+          const float v1 = (g0 + 2 * e2 + 1 >= first && g0 + 2 * e2 + 1 <= last) ? __uint_as_float(u[e2] & 0xffff0000u) : 0.f;
+          a = fmaf(w[2 * e2], v0, a);
+          a = fmaf(w[2 * e2 + 1], v1, a);
+        }
+      }
+      acc[i] = a;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
+#pragma unroll
+  for (int i = 0; i < DEC_DPL; ++i) {
+    const int d = lane + i * DA_WAVE;
+    if (d < D) part_acc[wave][d] = acc[i];
+  }
+  if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
+  __syncthreads();
+  // merge the wavefronts' partial softmaxes in a fixed order
+  float mm = part_m[0];
+#pragma unroll
+  for (int w2 = 1; w2 < DEC_WAVES; ++w2) mm = fmaxf(mm, part_m[w2]);
+  float ll = 0.f;
+  float f[DEC_WAVES];
+#pragma unroll
+  for (int w2 = 0; w2 < DEC_WAVES; ++w2) {
+    f[w2] = part_m[w2] == -INFINITY ? 0.f : expf(part_m[w2] - mm);
+    ll += part_l[w2] * f[w2];
+  }
+  const float inv = 1.0f / ll;
+  for (int d = t; d < D; d += DEC_WAVES * DA_WAVE) {
+    float o = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < DEC_WAVES; ++w2) o += part_acc[w2][d] * f[w2];
+    out[(size_t)s * out_ld + h * D + d] = f32_to_bf16(o * inv);
+  }
+}
+
+extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const int* block_table,
+                              int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
+                              float scale, int window, void* out, int out_ld, void* stream) {
+  DA_REQUIRE(S >= 0 && Hq > 0 && Hkv > 0 && page > 0, "attn_decode: bad sizes");
+  DA_REQUIRE(Hq % Hkv == 0, "attn_decode: %d query heads are not a multiple of %d key heads", Hq, Hkv);
+  DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= DEC_MAX_D, "attn_decode: head size %d is not a multiple of 16 up to %d", D, DEC_MAX_D);
+  DA_REQUIRE(page % 8 == 0 && DA_WAVE % page == 0, "attn_decode: page size %d must be 8, 16, 32 or 64", page);
+  DA_REQUIRE(q_ld >= Hq * D && out_ld >= Hq * D, "attn_decode: row lengths too small");
+  DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_decode: bad window or block table");
+  DA_REQUIRE((uintptr_t)cache % 16 == 0, "attn_decode: the cache must be 16-byte aligned");
+  if (S == 0) return 0;
+  const int pieces = D / 8;
+  dim3 grid(S * Hq), block(DEC_WAVES * DA_WAVE);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(C)                                                                                          \
+  hipLaunchKernelGGL(attn_decode_kernel<C>, grid, block, 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, \
+                     block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, (bf16_t*)out, out_ld)
+  if (pieces <= 2) LAUNCH(2);
+  else if (pieces <= 4) LAUNCH(4);
+  else if (pieces <= 8) LAUNCH(8);
+  else if (pieces <= 16) LAUNCH(16);
+  else LAUNCH(32);
+#undef LAUNCH
+  DA_CHECK_LAUNCH("attn_decode");
+  return 0;
+}

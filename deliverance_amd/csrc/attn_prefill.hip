@@ -1,0 +1,223 @@
+// Paged attention for prompt portions in bfloat16 on the matrix cores (flash-style: scores never
+// leave the chip).  A portion's rows sit at positions past .. past+T-1 of their sequence; row i
+// sees the keys lo_i .. past+i of the cache (earlier steps' keys and the portion's own, which were
+// written just before).
+//
+// One workgroup per (portion, query head, 128 query rows); 4 wavefronts of 32 rows each.  Keys
+// come in aligned tiles of 64 through LDS: the key rows as they lie in the pages, the values as
+// they lie in the pages too (dimension-major: a row of the LDS tile is one dimension, 64 keys).
+// Per tile and wavefront, with MFMA 32x32x16:
+//   S^T[key, row] = K . Q^T          keys are the MFMA's rows, so one lane holds ONE query row's
+//                                     scores for 16 keys: row maximum and sum need one exchange
+//                                     (lane ^ 32) instead of a reduction over the wavefront;
+//   online softmax in 32-bit (maximum, exp, sum, rescale: the recurrence of
+//   native/src/main/resources/decode_paged_attention_f32.wgsl:31-65);
+//   O^T[dim, row] += V^T . P^T       P^T is already in registers in the layout of the B operand
+//                                     (the matching, permuted order of keys is used for V^T).
+// Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:458-502.
+// A row's sums run over key tiles in ascending order starting at the aligned tile of its lo: the
+// order depends on the row's position (and window) only.
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+#define PF_WAVES 4
+#define PF_BQ 128          // query rows per workgroup
+#define PF_BK 64           // keys per tile
+#define PF_VLD (PF_BK + 8) // padded length of a value row in LDS
+
+template <int D16>         // head size / 16
+__global__ void __launch_bounds__(PF_WAVES * DA_WAVE)
+attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
+                    const int* __restrict__ block_table, int max_blocks,
+                    const int* __restrict__ q_start, const int* __restrict__ seq_lens, int seq0,
+                    int Hq, int Hkv, int page, float scale, int window,
+                    bf16_t* __restrict__ out, int out_ld) {
+  constexpr int D = D16 * 16;
+  constexpr int DT = (D + 31) / 32;       // 32-dimension tiles of the output
+  constexpr int KLD = D + 8;              // padded length of a key row in LDS
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BK * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[DT * 32 * PF_VLD];
+
+  const int s = seq0 + blockIdx.z, h = blockIdx.y;
+  const int row0 = q_start[s], T = q_start[s + 1] - row0;
+  const int i0 = blockIdx.x * PF_BQ;
+  if (i0 >= T) return;
+  const int past = seq_lens[s] - T;
+  const int hk = h / (Hq / Hkv);
+  const int* bt = block_table + (size_t)s * max_blocks;
+  const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
+  const int col = lane % 32, hf = lane / 32;
+
+  // this lane's query row (as a column of Q^T) and its position
+  const int qi = i0 + wave * 32 + col;
+  const bool q_ok = qi < T;
+  const int pq = past + qi;
+  const int q_lo = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
+  bf16x8_t qf[D16];
+#pragma unroll
+  for (int kd = 0; kd < D16; ++kd) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (q_ok) v = *(const uint4*)(q + (size_t)(row0 + qi) * q_ld + h * D + kd * 16 + hf * 8);
+    qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+  }
+  // the wavefront's rows span positions w_first .. w_last
+  const int w_first = past + i0 + wave * 32;
+  const int w_last_row = (i0 + wave * 32 + 31 < T - 1) ? i0 + wave * 32 + 31 : T - 1;
+  const bool wave_on = i0 + wave * 32 < T;
+  const int w_last = past + w_last_row;
+  const int w_lo = (window > 0 && w_first - window + 1 > 0) ? w_first - window + 1 : 0;
+  // the workgroup's keys
+  const int b_last = past + ((i0 + PF_BQ - 1 < T - 1) ? i0 + PF_BQ - 1 : T - 1);
+  const int b_lo = (window > 0 && past + i0 - window + 1 > 0) ? past + i0 - window + 1 : 0;
+
+  floatx16 acc_o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  for (int kt = (b_lo / PF_BK) * PF_BK; kt <= b_last; kt += PF_BK) {
+    // ---- stage the tile: keys kt .. kt+63, only those in b_lo .. b_last are read, the rest is zero
+    for (int c = t; c < PF_BK * (D / 8); c += PF_WAVES * DA_WAVE) {
+      const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (key >= b_lo && key <= b_last)
+        v = *(const uint4*)(cache + cache_k_row(bt[key / page], hk, key % page, Hkv, page, D) + pc * 8);
+      *(uint4*)&Ks[kr * KLD + pc * 8] = v;
+    }
+    for (int c = t; c < DT * 32 * (PF_BK / 8); c += PF_WAVES * DA_WAVE) {
+      const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;   // 8 keys of one dimension
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (d < D && key0 + 7 >= b_lo && key0 <= b_last) {
+        v = *(const uint4*)(cache + cache_v_base(bt[key0 / page], hk, Hkv, page, D) + (long long)d * page + key0 % page);
+        if (key0 < b_lo || key0 + 7 > b_last) {        // rows outside were never written for us
+          uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (key0 + e < b_lo || key0 + e > b_last) u[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
+          v = make_uint4(u[0], u[1], u[2], u[3]);
+        }
+      }
+      *(uint4*)&Vs[d * PF_VLD + g * 8] = v;
+    }
+    __syncthreads();
+
+    if (wave_on && kt <= w_last && kt + PF_BK - 1 >= w_lo) {
+      floatx16 sc[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[ks][r] = 0.f;
+#pragma unroll
+        for (int kd = 0; kd < D16; ++kd) {
+          const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ks[(ks * 32 + col) * KLD + kd * 16 + hf * 8]);
+          sc[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kd], sc[ks], 0, 0, 0);
+        }
+      }
+      // scale, mask, running maximum
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kt + ks * 32 + 8 * (r / 4) + 4 * hf + (r % 4);
+          const bool vis = q_ok && key <= pq && key >= q_lo;
+          const float v = vis ? sc[ks][r] * scale : -INFINITY;
+          sc[ks][r] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DA_WAVE));
+      const float m_new = fmaxf(m, tmax);
+      const bool any = m_new != -INFINITY;             // a row that has seen no key yet keeps zeros
+      const float alpha = any ? expf(m - m_new) : 1.f;
+      float tsum = 0.f;
+      bf16x8_t pf[2][2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          uint32_t u[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float p0 = any ? expf(sc[ks][kb * 8 + 2 * e] - m_new) : 0.f;
+            const float p1 = any ? expf(sc[ks][kb * 8 + 2 * e + 1] - m_new) : 0.f;
+            const bf16_t b0 = f32_to_bf16(p0), b1 = f32_to_bf16(p1);
+            // the sum uses the rounded weights, the same ones that multiply the values
+            tsum += bf16_to_f32(b0) + bf16_to_f32(b1);
+            u[e] = (uint32_t)b0 | ((uint32_t)b1 << 16);
+          }
+          pf[ks][kb] = __builtin_bit_cast(bf16x8_t, make_uint4(u[0], u[1], u[2], u[3]));
+        }
+      tsum += __shfl_xor(tsum, 32, DA_WAVE);
+      l = l * alpha + tsum;
+      m = m_new;
+#pragma unroll
+      for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] *= alpha;
+      // O^T += V^T . P^T ; the lane's 8 keys of a 16-key block are 4hf..4hf+3 and 8+4hf..8+4hf+3
+#pragma unroll
+      for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) {
+            const bf16_t* vr = &Vs[(i * 32 + col) * PF_VLD + ks * 32 + kb * 16 + 4 * hf];
+            const uint2 a0 = *(const uint2*)vr, a1 = *(const uint2*)(vr + 8);
+            const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a0.x, a0.y, a1.x, a1.y));
+            acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[ks][kb], acc_o[i], 0, 0, 0);
+          }
+    }
+    __syncthreads();
+  }
+
+  if (q_ok) {
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + (size_t)(row0 + qi) * out_ld + h * D;
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int d = i * 32 + 8 * r4 + 4 * hf;
+        if (d < D) {
+          uint32_t lo2 = (uint32_t)f32_to_bf16(acc_o[i][r4 * 4] * inv) | ((uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 1] * inv) << 16);
+          uint32_t hi2 = (uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 2] * inv) | ((uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 3] * inv) << 16);
+          *(uint2*)(orow + d) = make_uint2(lo2, hi2);
+        }
+      }
+  }
+}
+
+extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const int* block_table,
+                               int max_blocks, const int* q_start, const int* seq_lens, int seq0, int n_seqs,
+                               int max_query_len, int Hq, int Hkv, int D, int page, float scale, int window,
+                               void* out, int out_ld, void* stream) {
+  DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && page > 0 && max_query_len >= 0, "attn_prefill: bad sizes");
+  DA_REQUIRE(Hq % Hkv == 0, "attn_prefill: %d query heads are not a multiple of %d key heads", Hq, Hkv);
+  DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attn_prefill: head size %d is not a multiple of 16 up to 256", D);
+  DA_REQUIRE(page % 8 == 0 && PF_BK % page == 0, "attn_prefill: page size %d must be 8, 16, 32 or 64", page);
+  DA_REQUIRE(q_ld >= Hq * D && out_ld >= Hq * D && q_ld % 8 == 0 && out_ld % 4 == 0, "attn_prefill: row lengths");
+  DA_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)cache % 16 == 0) && ((uintptr_t)out % 8 == 0),
+             "attn_prefill: operands must be 16-byte aligned");
+  DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_prefill: bad window or block table");
+  DA_REQUIRE(n_seqs <= 65535 && Hq <= 65535, "attn_prefill: too many sequences or heads for one launch");
+  if (n_seqs == 0 || max_query_len == 0) return 0;
+  dim3 grid(da_ceil_div(max_query_len, PF_BQ), Hq, n_seqs), block(PF_WAVES * DA_WAVE);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(N)                                                                                         \
+  case N:                                                                                                 \
+    hipLaunchKernelGGL(attn_prefill_kernel<N>, grid, block, 0, st, (const bf16_t*)q, q_ld,                \
+                       (const bf16_t*)cache, block_table, max_blocks, q_start, seq_lens, seq0, Hq, Hkv,   \
+                       page, scale, window, (bf16_t*)out, out_ld);                                        \
+    break;
+  switch (D / 16) {
+    LAUNCH(1) LAUNCH(2) LAUNCH(3) LAUNCH(4) LAUNCH(5) LAUNCH(6) LAUNCH(7) LAUNCH(8)
+    LAUNCH(9) LAUNCH(10) LAUNCH(11) LAUNCH(12) LAUNCH(13) LAUNCH(14) LAUNCH(15) LAUNCH(16)
+  }
+#undef LAUNCH
+  DA_CHECK_LAUNCH("attn_prefill");
+  return 0;
+}

@@ -31,7 +31,6 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
   const int hk = h / (Hq / Hkv);
   const int p = positions[n];
   const int* bt = block_table + (size_t)seq_of_token[n] * max_blocks;
-  const long long page_elems = (long long)2 * Hkv * page * D;
 
   for (int d = lane; d < D; d += DA_WAVE) qs[d] = to_f32(q[(size_t)n * q_ld + h * D + d]);
   __syncthreads();
@@ -47,10 +46,10 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
     const bool valid = key <= p;
     float s = -INFINITY;
     if (valid) {
-      const long long base = (long long)bt[key / page] * page_elems;
+      const long long pg = bt[key / page];
       const int row = key % page;
-      const T* kr = cache + base + ((long long)hk * page + row) * D;
-      voff[lane] = base + ((long long)(Hkv + hk) * page + row) * D;
+      const T* kr = cache + cache_k_row(pg, hk, row, Hkv, page, D);
+      voff[lane] = cache_v_base(pg, hk, Hkv, page, D) + row;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
       s = dot * scale;
@@ -68,7 +67,7 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
       const int d = lane + i * DA_WAVE;
       if (d < D) {
         float a = acc[i] * alpha;
-        for (int j = 0; j < cnt; ++j) a = fmaf(ps[j], to_f32(cache[voff[j] + d]), a);
+        for (int j = 0; j < cnt; ++j) a = fmaf(ps[j], to_f32(cache[voff[j] + (long long)d * page]), a);
         acc[i] = a;
       }
     }

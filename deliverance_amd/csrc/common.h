@@ -105,4 +105,15 @@ __device__ __forceinline__ float apply_act(float x, int act) {
   }
 }
 
+// One cache slot is [n_pages][2][Hkv][page * D].  Keys of a (page, head) are page rows of D
+// ("row-major"); values are D runs of `page` ("dimension-major": the value of row r, dimension d
+// sits at d * page + r), which is the operand layout the matrix cores want for weights x values
+// and lets a decode lane own one dimension.
+__device__ __forceinline__ long long cache_k_row(long long page_id, int hk, int row, int Hkv, int page, int D) {
+  return page_id * (2LL * Hkv * page * D) + ((long long)hk * page + row) * D;
+}
+__device__ __forceinline__ long long cache_v_base(long long page_id, int hk, int Hkv, int page, int D) {
+  return page_id * (2LL * Hkv * page * D) + (long long)(Hkv + hk) * page * D;
+}
+
 static inline int da_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

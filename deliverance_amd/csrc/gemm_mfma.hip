@@ -1,0 +1,216 @@
+// bfloat16 matrix products on the gfx950 matrix cores, with the epilogues a block needs:
+//
+//   out[m, n] (+)= act( sum_k a[m, k] * w[n, k] + bias[n] )
+//
+// a: [M, K] bf16, w: [N, K] bf16 ("[out, in]", K contiguous), 32-bit accumulation; out is bf16,
+// or 32-bit (plain store or += for the residual stream).  Two kernels:
+//
+//  * gemm_tile: 128x128 block tile, 4 wavefronts of 64x64 (2x2 MFMA 32x32x16), operands staged
+//    through LDS with a register prefetch of the next K-slab.  For steps with many rows (prefill).
+//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its 4
+//    wavefronts split K, stream their part of w straight from memory into MFMA 16x16x32
+//    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
+//
+// In both, an output element sums over k in an order that depends on K only, never on M or on
+// the row's place in the batch.
+//
+// MFMA fragment layout (64 lanes).  32x32x16: lane l gives row (a) / column (b) l % 32 and the
+// 8 consecutive k starting at 8 * (l / 32); it receives, for r in 0..15, the element at
+// row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
+// l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define BM 128
+#define BN 128
+#define BKT 64               // k per slab
+#define LDS_LD (BKT + 8)     // padded row length in elements (144 bytes): spreads rows over banks
+
+struct Epilogue {
+  const void* bias;
+  int bias_dtype;
+  int act;
+  int accumulate;
+  void* out;
+  int out_dtype;
+  int ldo;
+};
+
+__device__ __forceinline__ void epilogue_store(const Epilogue& ep, int m, int n, float v, float bias) {
+  v = apply_act(v + bias, ep.act);
+  const size_t o = (size_t)m * ep.ldo + n;
+  if (ep.accumulate) ((float*)ep.out)[o] += v;
+  else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
+  else ((float*)ep.out)[o] = v;
+}
+
+__device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }
+
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
+                 Epilogue ep, int M, int N, int K, int tiles_m, int tiles_n) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * LDS_LD];
+
+  // Blocks that follow each other in launch order land on different XCDs (8 of them, each with
+  // its own L2).  Give each XCD a contiguous run of tiles, m fastest, so that the blocks of one
+  // XCD share slabs of w.
+  const int nblocks = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  {
+    const int per = nblocks / 8, rem = nblocks % 8;
+    const int xcd = pid % 8, local = pid / 8;
+    pid = xcd * per + (xcd < rem ? xcd : rem) + local;
+  }
+  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int wm = (wave % 2) * 64, wn = (wave / 2) * 64;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // each thread moves 4 chunks of 16 bytes of each operand per slab
+  uint4 ra[4], rw[4];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = t + 256 * i, row = c / 8, kc = (c % 8) * 8;
+      const bool kin = k0 + kc < K;
+      ra[i] = (kin && m0 + row < M) ? load16(a + (size_t)(m0 + row) * lda + k0 + kc) : zero;
+      rw[i] = (kin && n0 + row < N) ? load16(w + (size_t)(n0 + row) * ldw + k0 + kc) : zero;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = t + 256 * i, row = c / 8, kc = (c % 8) * 8;
+      *(uint4*)&As[row * LDS_LD + kc] = ra[i];
+      *(uint4*)&Ws[row * LDS_LD + kc] = rw[i];
+    }
+  };
+
+  const int fr = lane % 32, fk = (lane / 32) * 8;
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BKT) {
+    stash();
+    __syncthreads();
+    if (k0 + BKT < K) fetch(k0 + BKT);
+#pragma unroll
+    for (int kk = 0; kk < BKT; kk += 16) {
+      bf16x8_t af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        af[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&As[(wm + i * 32 + fr) * LDS_LD + kk + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        bf[j] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ws[(wn + j * 32 + fr) * LDS_LD + kk + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn + j * 32 + fr;
+    if (n >= N) continue;
+    const float b = ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (m < M) epilogue_store(ep, m, n, acc[i][j][r], b);
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// M <= 64.  Block: 16 columns of the output, all rows; wavefront v takes the k-chunks
+// v, v+4, v+8, ... of 32 elements each.
+// ---------------------------------------------------------------------------------------------
+#define SK_COLS 16
+template <int MT>   // row tiles of 16
+__global__ void __launch_bounds__(256)
+gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
+                   Epilogue ep, int M, int N, int K) {
+  __shared__ float red[4][MT * 16][SK_COLS + 1];
+  const int t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int n0 = blockIdx.x * SK_COLS;
+  const int fr = lane % 16, fk = (lane / 16) * 8;
+  floatx4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const bool wrow_ok = n0 + fr < N;
+  const bf16_t* wp = w + (size_t)(n0 + fr) * ldw + fk;
+  for (int k0 = wave * 32; k0 < K; k0 += 4 * 32) {
+    const bool kin = k0 + fk < K;
+    const uint4 wv = (wrow_ok && kin) ? load16(wp + k0) : zero;
+    const bf16x8_t bfrag = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int m = i * 16 + fr;
+      const uint4 av = (m < M && kin) ? load16(a + (size_t)m * lda + k0 + fk) : zero;
+      acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), bfrag, acc[i], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
+  __syncthreads();
+  for (int e = t; e < MT * 16 * SK_COLS; e += 256) {
+    const int m = e / SK_COLS, c = e % SK_COLS, n = n0 + c;
+    if (m < M && n < N) {
+      const float v = ((red[0][m][c] + red[1][m][c]) + red[2][m][c]) + red[3][m][c];
+      epilogue_store(ep, m, n, v, ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f);
+    }
+  }
+}
+
+extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
+                            int act, int accumulate, void* out, int out_dtype, int ldo, int M, int N, int K,
+                            void* stream) {
+  DA_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  DA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0,
+             "gemm_bf16: K, lda and ldw must be multiples of 8 (K=%d lda=%d ldw=%d)", K, lda, ldw);
+  DA_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
+  DA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_bf16: leading sizes too small");
+  DA_REQUIRE(!accumulate || out_dtype == DA_F32, "gemm_bf16: accumulation needs a 32-bit output");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16: unknown activation %d", act);
+  if (M == 0) return 0;
+  Epilogue ep{bias, bias_dtype, act, accumulate, out, out_dtype, ldo};
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* A = (const bf16_t*)a;
+  const bf16_t* W = (const bf16_t*)w;
+  if (M <= 64) {
+    dim3 grid(da_ceil_div(N, SK_COLS));
+    const int mt = da_ceil_div(M, 16);
+    if (mt == 1) hipLaunchKernelGGL(gemm_skinny_kernel<1>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
+    else if (mt == 2) hipLaunchKernelGGL(gemm_skinny_kernel<2>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
+    else if (mt == 3) hipLaunchKernelGGL(gemm_skinny_kernel<3>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
+    else hipLaunchKernelGGL(gemm_skinny_kernel<4>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
+  } else {
+    const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
+    hipLaunchKernelGGL(gemm_tile_kernel, dim3(tiles_m * tiles_n), dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K,
+                       tiles_m, tiles_n);
+  }
+  DA_CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}

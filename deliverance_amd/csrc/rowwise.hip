@@ -89,8 +89,9 @@ extern "C" int da_layernorm(const float* x, const int* rows, const void* w, int 
 // ------------------------------------------------------------------------------------------
 // Keys and values of the step's tokens go to their cache rows.
 // qkv: [N, ld] rows holding q | k | v; k starts at column k_off, v at v_off, each Hkv*D wide.
-// One cache slot (one layer's pages): [n_pages][2][Hkv][page][D]; slot_map[n] is
-// page_id * page + row, or -1 for a token whose keys are not kept.
+// One cache slot (one layer's pages): [n_pages][2][Hkv][page * D], keys row-major, values
+// dimension-major (see common.h); slot_map[n] is page_id * page + row, or -1 for a token whose
+// keys are not kept.
 // Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:315-336
 // ------------------------------------------------------------------------------------------
 template <typename T>
@@ -102,11 +103,11 @@ __global__ void kv_write_kernel(const T* __restrict__ qkv, int ld, int k_off, in
   if (slot < 0) return;
   const int pg = slot / page, row = slot % page;
   const int W = Hkv * D;
-  const size_t page_elems = (size_t)2 * Hkv * page * D;
   for (int i = threadIdx.x; i < 2 * W; i += blockDim.x) {
     const int kv = i / W, c = i % W, h = c / D, d = c % D;
     const T v = qkv[(size_t)n * ld + (kv ? v_off : k_off) + c];
-    cache[pg * page_elems + (((size_t)kv * Hkv + h) * page + row) * D + d] = v;
+    if (kv) cache[cache_v_base(pg, h, Hkv, page, D) + (long long)d * page + row] = v;
+    else cache[cache_k_row(pg, h, row, Hkv, page, D) + d] = v;
   }
 }
 

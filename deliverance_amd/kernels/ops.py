@@ -203,14 +203,97 @@ def kernel_mode() -> str:
     return _MODE
 
 
+def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
+    """out (+)= act(a @ w.T + bias) on the matrix cores; a, w bfloat16, K a multiple of 8."""
+    _dev(a, w, bias, out)
+    _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_mfma: a and w must be bfloat16")
+    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    _need(out.shape[0] == M and out.shape[1] == N, f"linear: out is {list(out.shape)}, expected [{M},{N}]")
+    _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
+    _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
+    _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
+    _check(build.load().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
+                                     _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
+                                     _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
+    return out
+
+
+def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
+            and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
-    """out (+)= act(a @ w.T + bias); picks the kernel by dtype and mode."""
+    """out (+)= act(a @ w.T + bias); picks the kernel by dtype and mode.  Shapes the matrix-core
+    kernel does not take (K not a multiple of 8) go to the plain kernel, which takes any."""
+    if _MODE == "tuned" and _mfma_ok(a, w):
+        return linear_mfma(a, w, bias, out, act, accumulate)
     return linear_ref(a, w, bias, out, act, accumulate)
+
+
+def _attn_common(q, cache_slot, block_table, n_heads, out, name):
+    _dev(q, cache_slot, block_table, out)
+    _rows_2d(q, "q"); _rows_2d(out, "out")
+    P, two, Hkv, page, D = cache_slot.shape
+    _need(cache_slot.is_contiguous() and two == 2, f"{name}: cache slot must be contiguous [pages,2,Hkv,page,D]")
+    _need(q.shape[1] == n_heads * D and out.shape[1] == n_heads * D, f"{name}: q/out must be [rows, Hq*D]")
+    _need(q.dtype == torch.bfloat16 and cache_slot.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+          f"{name}: q, cache and out must be bfloat16")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          f"{name}: block_table must be contiguous int32 [S, max_blocks]")
+    return Hkv, page, D
+
+
+def attention_decode(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
+                     seq_lens: torch.Tensor, n_seqs: int, n_heads: int, scale: float,
+                     window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+    """One query row per sequence: row s of q belongs to sequence s and sits at position
+    seq_lens[s] - 1."""
+    Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_decode")
+    _need(q.shape[0] >= n_seqs and out.shape[0] >= n_seqs and block_table.shape[0] >= n_seqs,
+          "attention_decode: fewer rows than sequences")
+    _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= n_seqs, "attention_decode: seq_lens must be int32 [S]")
+    _check(build.load().da_attn_decode(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+                                       block_table.shape[1], _ptr(seq_lens), n_seqs, n_heads, Hkv, D, page,
+                                       ctypes.c_float(scale), int(window or 0), _ptr(out), out.stride(0), _stream()))
+    return out
+
+
+def attention_prefill(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
+                      q_start: torch.Tensor, seq_lens: torch.Tensor, seq0: int, n_seqs: int,
+                      max_query_len: int, n_heads: int, scale: float, window: Optional[int],
+                      out: torch.Tensor) -> torch.Tensor:
+    """Portions: sequence s (seq0 <= s < seq0 + n_seqs) owns rows q_start[s] .. q_start[s+1]-1 of q
+    and out; its last row sits at position seq_lens[s] - 1."""
+    Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_prefill")
+    _need(q_start.dtype == torch.int32 and q_start.numel() >= seq0 + n_seqs + 1, "attention_prefill: q_start must be int32 [S+1]")
+    _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= seq0 + n_seqs, "attention_prefill: seq_lens must be int32 [S]")
+    _need(block_table.shape[0] >= seq0 + n_seqs, "attention_prefill: block table has fewer rows than sequences")
+    _need(q.shape[0] == out.shape[0], "attention_prefill: q and out differ in rows")
+    _check(build.load().da_attn_prefill(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+                                        block_table.shape[1], _ptr(q_start), _ptr(seq_lens), seq0, n_seqs,
+                                        max_query_len, n_heads, Hkv, D, page, ctypes.c_float(scale),
+                                        int(window or 0), _ptr(out), out.stride(0), _stream()))
+    return out
 
 
 def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int,
                     scale: float, window: Optional[int], out: torch.Tensor) -> torch.Tensor:
-    """Attention of every row of the step over its sequence's pages."""
-    return attention_ref(q, cache_slot, ctx.block_tables[group], ctx.seq_of_token, ctx.positions,
-                         n_heads, scale, window, out)
+    """Attention of every row of the step over its sequence's pages.  In bfloat16 the one-token
+    sequences (the first ``ctx.n_decode``) go to the decode kernel and the portions to the
+    prefill kernel; 32-bit and the reference mode use the plain kernel for all rows."""
+    bt = ctx.block_tables[group]
+    if _MODE == "tuned" and q.dtype == torch.bfloat16:
+        nd = ctx.n_decode
+        if nd:
+            attention_decode(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, out)
+        if ctx.n_seqs > nd:
+            attention_prefill(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
+                              ctx.max_query_len, n_heads, scale, window, out)
+        return out
+    return attention_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, scale, window, out)

@@ -1,0 +1,362 @@
+"""Each kernel alone against a plain reference, at other sizes than the engine's tiny models
+use: sizes that are no power of two, head sizes in steps of 16, grouped heads, windows, pages
+scattered over the pool, and a pool that is NaN wherever nothing was written."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_gpt2 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from deliverance_amd.kernels import ops as o
+    return o
+
+
+def bf(x):
+    return x.to(torch.bfloat16)
+
+
+# ----------------------------------------------------------------------------- embedding, norm
+@pytest.mark.parametrize("table_dtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, table_dtype):
+    g = torch.Generator().manual_seed(0)
+    V, Pn, E, N = 1000, 77, 200, 37
+    wte = torch.randn(V, E, generator=g).to(table_dtype).to(DEV)
+    wpe = torch.randn(Pn, E, generator=g).to(table_dtype).to(DEV)
+    tok = torch.randint(0, V, (N,), generator=g, dtype=torch.int32).to(DEV)
+    pos = torch.randint(0, Pn, (N,), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.empty(N, E, device=DEV)
+    ops.embed(tok, pos, wte, wpe, out)
+    want = wte.float()[tok.long()] + wpe.float()[pos.long()]
+    assert torch.equal(out, want)
+    ops.embed(tok, pos, wte, None, out)
+    assert torch.equal(out, wte.float()[tok.long()])
+
+
+@pytest.mark.parametrize("E,eps", [(7, 1e-5), (200, 1e-6), (1600, 1e-5), (64, 1e-1)])
+def test_layernorm(ops, E, eps):
+    g = torch.Generator().manual_seed(1)
+    N = 19
+    x = (torch.randn(N, E, generator=g) * 3 + 5).to(DEV)       # a large mean: E[x^2]-mean^2 would lose digits
+    w, b = torch.randn(E, generator=g).to(DEV), torch.randn(E, generator=g).to(DEV)
+    out = torch.empty(N, E, device=DEV)
+    ops.layernorm(x, w, b, eps, out)
+    want = F.layer_norm(x.double(), (E,), w.double(), b.double(), eps)
+    assert (out.double() - want).abs().max() < 2e-5
+    # bfloat16 parameters and output, gathered rows
+    rows = torch.tensor([5, 0, 18, 5], dtype=torch.int32, device=DEV)
+    o2 = torch.empty(4, E, device=DEV, dtype=torch.bfloat16)
+    ops.layernorm(x, bf(w), bf(b), eps, o2, rows)
+    want2 = F.layer_norm(x.double(), (E,), bf(w).double(), bf(b).double(), eps)[rows.long()]
+    assert (o2.double() - want2).abs().max() < 4e-2
+    assert torch.equal(o2[0], o2[3])
+    if E == 7:   # the reference's own vector (LayerNormTest.java:40,51,77,88)
+        xv = torch.tensor([[-1.1151, 0.1490, -1.0923, -1.4551, 1.3358, 0.3075, 0.6278]], device=DEV)
+        o3 = torch.empty(1, 7, device=DEV)
+        ops.layernorm(xv, torch.ones(7, device=DEV), torch.zeros(7, device=DEV), 1e-5, o3)
+        want3 = torch.tensor([-0.9635, 0.3355, -0.9401, -1.3129, 1.5551, 0.4984, 0.8275], device=DEV)
+        assert (o3[0] - want3).abs().max() < 1e-4
+
+
+# ----------------------------------------------------------------------------- products
+def _gemm_case(ops, fn, M, N, K, dtype, act, accumulate, bias, out_dtype, g):
+    a = (torch.randn(M, K, generator=g) * 0.5).to(dtype).to(DEV)
+    w = (torch.randn(N, K, generator=g) * 0.2).to(dtype).to(DEV)
+    b = torch.randn(N, generator=g).to(dtype).to(DEV) if bias else None
+    base = torch.randn(M, N, generator=g).to(DEV)
+    out = base.clone() if accumulate else torch.empty(M, N, device=DEV, dtype=out_dtype)
+    fn(a, w, b, out, act, accumulate)
+    ref = a.double() @ w.double().t()
+    if bias:
+        ref = ref + b.double()
+    if act == "gelu_new":
+        ref = F.gelu(ref, approximate="tanh")
+    elif act == "gelu":
+        ref = F.gelu(ref)
+    elif act == "relu":
+        ref = F.relu(ref)
+    elif act == "silu":
+        ref = F.silu(ref)
+    if accumulate:
+        ref = ref + base.double()
+    return out.double(), ref
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 50, 24), (5, 1000, 96), (70, 200, 96), (130, 77, 200), (64, 64, 64)])
+def test_gemm_plain_32bit(ops, M, N, K):
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    for act, acc, bias in ((None, False, True), ("gelu_new", False, True), ("gelu", False, False),
+                           (None, True, True), ("silu", False, True), ("relu", False, True)):
+        out, ref = _gemm_case(ops, ops.linear_ref, M, N, K, torch.float32, act, acc, bias, torch.float32, g)
+        assert (out - ref).abs().max() < 2e-5 * max(1.0, ref.abs().max().item())
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 40, 64, 65, 128, 200, 513])
+@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24)])
+def test_gemm_matrix_cores(ops, M, N, K):
+    g = torch.Generator().manual_seed(M * 7 + N)
+    for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
+                               (None, True, True, torch.float32), (None, False, False, torch.float32),
+                               ("gelu", False, True, torch.bfloat16)):
+        out, ref = _gemm_case(ops, ops.linear_mfma, M, N, K, torch.bfloat16, act, acc, bias, od, g)
+        tol = (1e-2 if od == torch.bfloat16 else 1e-4) * max(1.0, ref.abs().max().item())
+        assert (out - ref).abs().max() < tol, (act, acc, bias, od)
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    """A row's result is the same whatever other rows share the call (within one kernel)."""
+    g = torch.Generator().manual_seed(3)
+    K, N = 768, 300
+    a = bf(torch.randn(200, K, generator=g)).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
+    full = torch.empty(200, N, device=DEV, dtype=torch.bfloat16)
+    ops.linear_mfma(a, w, None, full)
+    part = torch.empty(90, N, device=DEV, dtype=torch.bfloat16)
+    ops.linear_mfma(a[60:150].contiguous(), w, None, part)
+    assert torch.equal(part, full[60:150])
+    small = torch.empty(64, N, device=DEV, dtype=torch.bfloat16)
+    ops.linear_mfma(a[:64].contiguous(), w, None, small)
+    one = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
+    ops.linear_mfma(a[10:11].contiguous(), w, None, one)
+    assert torch.equal(one[0], small[10])
+
+
+def test_gemm_refuses_what_it_cannot_take(ops):
+    a = torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(8, 12, device=DEV, dtype=torch.bfloat16)
+    out = torch.zeros(4, 8, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="multiples of 8"):
+        ops.linear_mfma(a, w, None, out)
+    ops.linear(a, w, None, out)                     # the dispatcher sends it to the plain kernel
+    with pytest.raises(ops.KernelError):
+        ops.linear_ref(a, w, None, torch.zeros(4, 9, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(ops.KernelError, match="float32 output"):
+        ops.linear_ref(a, w, None, out, None, True)
+
+
+# ----------------------------------------------------------------------------- paged attention
+class PagedCase:
+    """Sequences with their keys and values scattered over a NaN-filled pool."""
+
+    def __init__(self, lens, new, Hq, Hkv, D, page, dtype, seed, scale_boost=None):
+        g = torch.Generator().manual_seed(seed)
+        self.lens, self.new, self.Hq, self.Hkv, self.D, self.page = lens, new, Hq, Hkv, D, page
+        S = len(lens)
+        n_pages = sum(-(-n // page) for n in lens) + 5
+        perm = torch.randperm(n_pages, generator=g).tolist()
+        self.cache = torch.full((n_pages, 2, Hkv, page, D), float("nan"), dtype=dtype, device=DEV)
+        max_blocks = max(-(-n // page) for n in lens)
+        bt = torch.full((S, max_blocks), -1, dtype=torch.int32)
+        self.k, self.v, self.q = [], [], []
+        for s, n in enumerate(lens):
+            k = torch.randn(n, Hkv * D, generator=g).to(dtype)
+            v = torch.randn(n, Hkv * D, generator=g).to(dtype)
+            q = torch.randn(new[s], Hq * D, generator=g).to(dtype)
+            if scale_boost is not None:      # one far key stands out for the last query
+                far, boost = scale_boost
+                q[-1] *= boost
+                qv = q[-1].float().view(Hq, D)[:: Hq // Hkv]
+                k[far] = (qv / qv.norm(dim=1, keepdim=True) * 8.0).reshape(-1).to(dtype)
+            self.k.append(k); self.v.append(v); self.q.append(q)
+            for j in range(-(-n // page)):
+                bt[s, j] = perm.pop()
+        self.bt = bt.to(DEV)
+        # fill through the engine's own write kernel
+        from deliverance_amd.kernels import ops as o
+        for s, n in enumerate(lens):
+            qkv = torch.cat([torch.zeros(n, Hq * D, dtype=dtype), self.k[s], self.v[s]], dim=1).to(DEV)
+            slots = torch.tensor([int(bt[s, pos // page]) * page + pos % page for pos in range(n)], dtype=torch.int32, device=DEV)
+            o.kv_write(qkv, Hq * D, Hq * D + Hkv * D, self.cache, slots, Hkv, D)
+        self.qcat = torch.cat(self.q).to(DEV)
+        starts = np.cumsum([0] + list(new))
+        self.q_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+        self.seq_lens = torch.tensor(lens, dtype=torch.int32, device=DEV)
+        self.seq_of = torch.tensor([s for s, n in enumerate(new) for _ in range(n)], dtype=torch.int32, device=DEV)
+        self.pos = torch.tensor([lens[s] - new[s] + i for s in range(S) for i in range(new[s])], dtype=torch.int32, device=DEV)
+
+    def plain(self, scale, window):
+        outs = []
+        for s in range(len(self.lens)):
+            o = P.causal_attention(self.q[s].double().numpy(), self.k[s].double().numpy(), self.v[s].double().numpy(),
+                                   self.Hq, scale, window=window, n_kv_head=self.Hkv, past=self.lens[s] - self.new[s])
+            outs.append(o)
+        return np.concatenate(outs)
+
+
+ATT_TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+                                                  (3, 3, 128, 64, None), (5, 5, 64, 16, 100)])
+def test_attention_plain_kernel(ops, dtype, Hq, Hkv, D, page, window):
+    case = PagedCase(lens=[70, 5, 131, 64], new=[70, 1, 9, 2], Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=dtype, seed=D)
+    out = torch.empty_like(case.qcat)
+    scale = 0.7 / math.sqrt(D)
+    ops.attention_ref(case.qcat, case.cache, case.bt, case.seq_of, case.pos, Hq, scale, window, out)
+    assert np.abs(out.double().cpu().numpy() - case.plain(scale, window)).max() < ATT_TOL[dtype]
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+                                                  (3, 3, 128, 64, None), (12, 12, 64, 16, None), (5, 5, 64, 16, 100),
+                                                  (2, 2, 256, 16, None), (25, 25, 64, 32, 70)])
+def test_attention_decode_kernel(ops, Hq, Hkv, D, page, window):
+    lens = [1, 2, 63, 64, 65, 300, 129, 17, 1000]
+    case = PagedCase(lens=lens, new=[1] * len(lens), Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + 1)
+    out = torch.empty_like(case.qcat)
+    scale = 0.7 / math.sqrt(D)
+    ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, out)
+    got = out.double().cpu().numpy()
+    assert np.isfinite(got).all()
+    assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+                                                  (3, 3, 128, 64, None), (12, 12, 64, 16, None), (5, 5, 64, 16, 100),
+                                                  (2, 2, 256, 16, None), (2, 2, 240, 16, None), (3, 1, 64, 32, 200)])
+def test_attention_prefill_kernel(ops, Hq, Hkv, D, page, window):
+    lens = [70, 200, 131, 64, 2, 300, 513]
+    new = [70, 9, 131, 2, 2, 129, 260]            # whole prompts, short portions after a long past, tiles' edges
+    case = PagedCase(lens=lens, new=new, Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + 2)
+    out = torch.full_like(case.qcat, float("nan"))
+    scale = 0.7 / math.sqrt(D)
+    ops.attention_prefill(case.qcat, case.cache, case.bt, case.q_start, case.seq_lens, 0, len(lens), max(new), Hq,
+                          scale, window, out)
+    got = out.double().cpu().numpy()
+    assert np.isfinite(got).all()
+    assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
+
+
+def test_attention_reference_vector_shape(ops):
+    """The shape of the reference's own paged-attention test: 4 query heads on 2 key heads, head 8
+    there (16 here: head sizes come in steps of 16), pages of 3 rows there (16 here), 5 visible rows,
+    scale 0.25, inputs by its closed formula (tensor/src/test/java/io/teknek/deliverance/tensor/
+    operations/TensorOperationsDecodePagedAttentionTest.java:18-47,92-99)."""
+    Hq, Hkv, D, page, rows = 4, 2, 16, 16, 5
+
+    def tensor(r, c, seed):
+        return torch.tensor([[(((i * 19 + j * 23 + seed) % 43) - 21) / 21.0 for j in range(c)] for i in range(r)])
+    q = tensor(1, Hq * D, 3)
+    k = torch.cat([tensor(3, Hkv * D, 7), tensor(3, Hkv * D, 11)])[:rows]
+    v = torch.cat([tensor(3, Hkv * D, 13), tensor(3, Hkv * D, 17)])[:rows]
+    want = P.causal_attention(q.double().numpy(), k.double().numpy(), v.double().numpy(), Hq, 0.25, n_kv_head=Hkv, past=rows - 1)
+    for dtype in (torch.float32, torch.bfloat16):
+        cache = torch.full((2, 2, Hkv, page, D), float("nan"), dtype=dtype, device=DEV)
+        qkv = torch.cat([torch.zeros(rows, Hq * D), k, v], dim=1).to(dtype).to(DEV)
+        slots = torch.tensor([16 + i for i in range(rows)], dtype=torch.int32, device=DEV)     # page 1
+        ops.kv_write(qkv, Hq * D, Hq * D + Hkv * D, cache, slots, Hkv, D)
+        bt = torch.tensor([[1]], dtype=torch.int32, device=DEV)
+        qd = q.to(dtype).to(DEV)
+        out = torch.empty_like(qd)
+        ops.attention_ref(qd, cache, bt, torch.zeros(1, dtype=torch.int32, device=DEV),
+                          torch.tensor([rows - 1], dtype=torch.int32, device=DEV), Hq, 0.25, None, out)
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        assert np.abs(out.double().cpu().numpy() - want).max() < tol
+        if dtype == torch.bfloat16:
+            out2 = torch.empty_like(qd)
+            ops.attention_decode(qd, cache, bt, torch.tensor([rows], dtype=torch.int32, device=DEV), 1, Hq, 0.25, None, out2)
+            assert np.abs(out2.double().cpu().numpy() - want).max() < tol
+
+
+def test_a_far_key_among_hundreds_is_found(ops):
+    """Random keys give near-uniform weights, which would hide a lost key: here one key far back
+    carries almost all the weight of the last query."""
+    for far, n in ((3, 700), (255, 700), (256, 700), (639, 700)):
+        case = PagedCase(lens=[n], new=[1], Hq=2, Hkv=2, D=64, page=16, dtype=torch.bfloat16, seed=far, scale_boost=(far, 3.0))
+        scale = 1 / 8
+        want = case.plain(scale, None)
+        # the weight of the far key dominates: the result is close to that key's value
+        assert np.abs(want[0, :64] - case.v[0][far, :64].double().numpy()).max() < 0.2
+        out = torch.empty_like(case.qcat)
+        ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, 1, 2, scale, None, out)
+        assert np.abs(out.double().cpu().numpy() - want).max() < 2e-2
+        case2 = PagedCase(lens=[n], new=[130], Hq=2, Hkv=2, D=64, page=16, dtype=torch.bfloat16, seed=far, scale_boost=(far, 3.0))
+        out2 = torch.empty_like(case2.qcat)
+        ops.attention_prefill(case2.qcat, case2.cache, case2.bt, case2.q_start, case2.seq_lens, 0, 1, 130, 2, scale, None, out2)
+        assert np.abs(out2.double().cpu().numpy() - case2.plain(scale, None)).max() < 2e-2
+
+
+# ----------------------------------------------------------------------------- sampling
+def _records(params_list, V, seeds):
+    import struct
+    from deliverance_amd.sampling import JavaRandom, device_record
+    words, us = [], []
+    for p, seed in zip(params_list, seeds):
+        rng = JavaRandom(seed)
+        rec = device_record(p, rng, V)
+        words += struct.unpack("<8i", rec)
+        us.append(struct.unpack("<fififfii", rec)[4])
+    return torch.tensor(words, dtype=torch.int32, device=DEV), us
+
+
+def test_sampling_kernel_against_the_plain_sampler(ops):
+    from deliverance_amd.sampling import GeneratorParameters as GP
+    g = torch.Generator().manual_seed(5)
+    V = 50257
+    combos = [GP(), GP(temperature=0.8), GP(temperature=1.3, top_k=50), GP(temperature=0.7, top_p=0.9),
+              GP(temperature=1.0, top_k=40, top_p=0.95), GP(temperature=1.0, top_k=0.999), GP(temperature=2.0, top_p=0.3),
+              GP(temperature=0.9, top_k=5, top_p=0.5, uniform_top_p=1.0), GP(temperature=1.0, top_p=1.0)]
+    rows, plist, seeds = [], [], []
+    for i in range(4):
+        for c in combos:
+            rows.append(torch.randn(V, generator=g) * 3.0)
+            plist.append(c); seeds.append(100 + i)
+    logits = torch.stack(rows).to(DEV)
+    rec, us = _records(plist, V, seeds)
+    out = torch.empty(len(rows), dtype=torch.int32, device=DEV)
+    ops.sample(logits, rec, out)
+    got = out.cpu().tolist()
+    for r, (p, u) in enumerate(zip(plist, us)):
+        lg = rows[r].numpy()
+        want = int(np.argmax(lg)) if p.temperature == 0 else \
+            P.sample_top_k_top_p(lg, p.temperature, p.top_k, p.top_p, p.uniform_top_p, u)
+        assert got[r] == want, (r, p)
+
+
+def test_sampling_vectors_of_the_reference(ops):
+    """core/src/test/java/io/teknek/deliverance/model/TopKSamplerTest.java:23-54, with the draws given."""
+    import struct
+    logits = torch.tensor([[5.0, 4.0, 3.0, 2.0, 1.0]] * 5 + [[1.0, 1.0, 1.0, 0.0, 1.0]] * 2, device=DEV)
+
+    def rec(T, k, p, uni, u):
+        return struct.unpack("<8i", struct.pack("<fififfii", T, k, p, uni, u, 0.0, 0, 0))
+    words = (rec(1.0, 2, 0.95, 0, 0.99) + rec(1.0, 2, 0.95, 0, 0.60) + rec(1.0, 2, 0.95, 1, 0.60) + rec(0.0, 0, 0.0, 0, 0.0)
+             + rec(1.0, 0, 0.0, 0, 0.999999) + rec(0.0, 0, 0.0, 0, 0.0) + rec(1.0, 3, 0.0, 0, 0.70))
+    out = torch.empty(7, dtype=torch.int32, device=DEV)
+    ops.sample(logits, torch.tensor(words, dtype=torch.int32, device=DEV), out)
+    # weighted 0.99 -> 1, weighted 0.60 -> 0, uniform in nucleus 0.60 -> 1, greedy -> 0, u ~ 1 -> last token,
+    # greedy ties -> lowest index, top-3 of equal logits keeps indices 0,1,2 and 0.70 lands on the third
+    assert out.cpu().tolist() == [1, 0, 1, 0, 4, 0, 2]
+
+
+def test_xtc_and_logprobs(ops):
+    import struct
+    V = 1000
+    g = torch.Generator().manual_seed(9)
+    lg = torch.randn(V, generator=g)
+    lg[10], lg[20], lg[30] = 9.0, 8.5, 8.0          # three tokens above a 10% threshold
+    logits = torch.stack([lg, lg, lg]).to(DEV)
+
+    def rec(T, thr, active):
+        return struct.unpack("<8i", struct.pack("<fififfii", T, 0, 0.0, 0, 0.0, thr, active, 0))
+    words = rec(0.0, 0.1, 1) + rec(0.0, 0.1, 0) + rec(1.0, 0.1, 1)
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    params = torch.tensor(words, dtype=torch.int32, device=DEV)
+    ops.sample(logits, params, out)
+    # active: the least likely of the tokens above the threshold; inactive: the maximum
+    assert out.cpu().tolist() == [30, 10, 30]
+    idx = torch.empty(3, 4, dtype=torch.int32, device=DEV)
+    lp = torch.empty(3, 4, dtype=torch.float32, device=DEV)
+    ops.top_logprobs(logits, params, 4, idx, lp)
+    want = torch.log_softmax(lg.double(), 0)
+    top = torch.topk(want, 4)
+    assert idx[0].cpu().tolist() == top.indices.tolist()
+    assert (lp[0].cpu().double() - top.values).abs().max() < 1e-4
