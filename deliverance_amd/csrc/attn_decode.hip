@@ -1,7 +1,9 @@
 // Paged attention for decode rows in bfloat16: one query row per sequence.
 //
-// One workgroup of 4 wavefronts per (sequence, query head).  The keys lo..p of the sequence
-// are walked in aligned chunks of 64; wavefront v takes chunks v, v+4, ...
+// One workgroup of 16 wavefronts per (sequence, query head).  The keys lo..p of the sequence
+// are walked in aligned chunks of 64; wavefront v takes chunks v, v+16, ... (one each up to a
+// context of 1,024).  All loads of a phase are issued before any is used, so a chunk costs two
+// memory round trips.
 //   scores : CPR lanes share a key, each holding a 16-byte piece of the key row and the matching
 //            piece of q in registers; their partial dot products are added by lane exchange.
 //            One load instruction so covers 64 / CPR whole key rows that lie next to each other.
@@ -9,19 +11,19 @@
 //            (the recurrence of native/src/main/resources/decode_paged_attention_f32.wgsl:31-65).
 //   values : values are stored dimension-major, so lane d reads 8 consecutive keys of its own
 //            dimension in 16 bytes and keeps one accumulator; no exchange between lanes.
-// The four wavefronts' partial results are merged in LDS in a fixed order.  Every sum's order
+// The wavefronts' partial results are merged in LDS in a fixed order.  Every sum's order
 // depends on p and lo only, never on the batch.
 //
 // Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:504-532;
 // tensor/src/main/java/io/teknek/deliverance/tensor/operations/TensorOperations.java:240-272.
 #include "common.h"
+#include <stdlib.h>
 
-#define DEC_WAVES 4
 #define DEC_MAX_D 256
 #define DEC_DPL (DEC_MAX_D / DA_WAVE)   // value dimensions per lane at most
 
 // CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
-template <int CPR>
+template <int CPR, int DEC_WAVES>
 __global__ void __launch_bounds__(DEC_WAVES * DA_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                    const int* __restrict__ block_table, int max_blocks,
@@ -42,9 +44,15 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   const int piece = lane % CPR, sub = lane / CPR;
   const bool piece_ok = piece * 8 < D;
   float qf[8];
+  {
+    const uint4 qv = *(const uint4*)(q + (size_t)s * q_ld + h * D + (piece_ok ? piece * 8 : 0));
+    const uint32_t u[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    qf[e] = piece_ok ? bf16_to_f32(q[(size_t)s * q_ld + h * D + piece * 8 + e]) * scale : 0.f;
+    for (int e = 0; e < 4; ++e) {
+      qf[2 * e] = piece_ok ? __uint_as_float(u[e] << 16) * scale : 0.f;
+      qf[2 * e + 1] = piece_ok ? __uint_as_float(u[e] & 0xffff0000u) * scale : 0.f;
+    }
+  }
 
   float acc[DEC_DPL];
 #pragma unroll
@@ -52,22 +60,28 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   float m = -INFINITY, l = 0.f;
 
   for (int c0 = (lo / DA_WAVE) * DA_WAVE + wave * DA_WAVE; c0 <= p; c0 += DEC_WAVES * DA_WAVE) {
-    // ---- scores: iteration i handles keys c0 + i*G + sub
+    // ---- scores: iteration i handles keys c0 + i*G + sub; all loads first, then the arithmetic
     float mine = -INFINITY;      // one key's score per lane, once the loop is done
+    uint4 kv[CPR];
+    const int safe_key = p;      // a row that surely exists, read in place of rows that are not seen
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
       const int key = c0 + i * G + sub;
       const bool valid = key >= lo && key <= p;
-      float dot = 0.f;
-      if (valid && piece_ok) {
-        const bf16_t* kr = cache + cache_k_row(bt[key / page], hk, key % page, Hkv, page, D) + piece * 8;
-        const uint4 kv = *(const uint4*)kr;
-        const uint32_t u[4] = {kv.x, kv.y, kv.z, kv.w};
+      const int kk = valid ? key : safe_key;
+      const bf16_t* kr = cache + cache_k_row(bt[kk / page], hk, kk % page, Hkv, page, D) + (piece_ok ? piece * 8 : 0);
+      kv[i] = *(const uint4*)kr;
+    }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          dot = fmaf(qf[2 * e], __uint_as_float(u[e] << 16), dot);
-          dot = fmaf(qf[2 * e + 1], __uint_as_float(u[e] & 0xffff0000u), dot);
-        }
+    for (int i = 0; i < CPR; ++i) {
+      const int key = c0 + i * G + sub;
+      const bool valid = key >= lo && key <= p;
+      const uint32_t u[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        dot = fmaf(qf[2 * e], __uint_as_float(u[e] << 16), dot);
+        dot = fmaf(qf[2 * e + 1], __uint_as_float(u[e] & 0xffff0000u), dot);
       }
 #pragma unroll
       for (int o = 1; o < CPR; o <<= 1) dot += __shfl_xor(dot, o, DA_WAVE);
@@ -94,12 +108,22 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       const int d = lane + i * DA_WAVE;
       if (d >= D) break;
       float a = acc[i] * alpha;
-      for (int g0 = (first / 8) * 8; g0 <= last; g0 += 8) {   // groups of 8 keys, never across a page
-        const bf16_t* vr = cache + cache_v_base(bt[g0 / page], hk, Hkv, page, D) + (long long)d * page + g0 % page;
-        const uint4 vv = *(const uint4*)vr;
-        const uint32_t u[4] = {vv.x, vv.y, vv.z, vv.w};
-        const float4 w0 = *(const float4*)&ps[wave][g0 - c0];
-        const float4 w1 = *(const float4*)&ps[wave][g0 - c0 + 4];
+      // the chunk's 8 groups of 8 keys (a group never crosses a page); groups with no seen key
+      // read the group of `last` instead and are dropped
+      uint4 vv[8];
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const int g0 = c0 + g * 8;
+        const bool any = g0 + 7 >= first && g0 <= last;
+        const int gs = any ? g0 : (last / 8) * 8;
+        vv[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+      }
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const int g0 = c0 + g * 8;
+        const uint32_t u[4] = {vv[g].x, vv[g].y, vv[g].z, vv[g].w};
+        const float4 w0 = *(const float4*)&ps[wave][g * 8];
+        const float4 w1 = *(const float4*)&ps[wave][g * 8 + 4];
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
@@ -134,7 +158,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     f[w2] = part_m[w2] == -INFINITY ? 0.f : expf(part_m[w2] - mm);
     ll += part_l[w2] * f[w2];
   }
-  const float inv = 1.0f / ll;
+  const float inv = ll > 0.f ? 1.0f / ll : 0.f;     // a sequence of length 0 (padding) gives zeros
   for (int d = t; d < D; d += DEC_WAVES * DA_WAVE) {
     float o = 0.f;
 #pragma unroll
@@ -152,20 +176,31 @@ extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const 
   DA_REQUIRE(page % 8 == 0 && DA_WAVE % page == 0, "attn_decode: page size %d must be 8, 16, 32 or 64", page);
   DA_REQUIRE(q_ld >= Hq * D && out_ld >= Hq * D, "attn_decode: row lengths too small");
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_decode: bad window or block table");
-  DA_REQUIRE((uintptr_t)cache % 16 == 0, "attn_decode: the cache must be 16-byte aligned");
+  DA_REQUIRE((uintptr_t)cache % 16 == 0 && (uintptr_t)q % 16 == 0 && q_ld % 8 == 0,
+             "attn_decode: q and the cache must be 16-byte aligned");
   if (S == 0) return 0;
   const int pieces = D / 8;
-  dim3 grid(S * Hq), block(DEC_WAVES * DA_WAVE);
+  static int waves = -1;
+  if (waves < 0) { const char* e = getenv("DA_DECODE_WAVES"); waves = e ? atoi(e) : 8; }
+  dim3 grid(S * Hq);
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(C)                                                                                          \
-  hipLaunchKernelGGL(attn_decode_kernel<C>, grid, block, 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, \
-                     block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, (bf16_t*)out, out_ld)
+#define LAUNCH2(C, W)                                                                                      \
+  hipLaunchKernelGGL((attn_decode_kernel<C, W>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld,   \
+                     (const bf16_t*)cache, block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, \
+                     (bf16_t*)out, out_ld)
+#define LAUNCH(C)                                                  \
+  do {                                                             \
+    if (waves == 16) LAUNCH2(C, 16);                               \
+    else if (waves == 4) LAUNCH2(C, 4);                            \
+    else LAUNCH2(C, 8);                                            \
+  } while (0)
   if (pieces <= 2) LAUNCH(2);
   else if (pieces <= 4) LAUNCH(4);
   else if (pieces <= 8) LAUNCH(8);
   else if (pieces <= 16) LAUNCH(16);
   else LAUNCH(32);
 #undef LAUNCH
+#undef LAUNCH2
   DA_CHECK_LAUNCH("attn_decode");
   return 0;
 }

@@ -43,7 +43,8 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
 
   for (int c0 = lo; c0 <= p; c0 += DA_WAVE) {
     const int key = c0 + lane;
-    const bool valid = key <= p;
+    // a row whose sequence has no page there (a padding row of a fixed-shape step) sees nothing
+    const bool valid = key <= p && bt[key / page] >= 0;
     float s = -INFINITY;
     if (valid) {
       const long long pg = bt[key / page];
@@ -67,13 +68,16 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
       const int d = lane + i * DA_WAVE;
       if (d < D) {
         float a = acc[i] * alpha;
-        for (int j = 0; j < cnt; ++j) a = fmaf(ps[j], to_f32(cache[voff[j] + (long long)d * page]), a);
+        for (int j = 0; j < cnt; ++j) {
+          const float pj = ps[j];                  // 0 for a key that is not seen: its row is not read
+          if (pj != 0.f) a = fmaf(pj, to_f32(cache[voff[j] + (long long)d * page]), a);
+        }
         acc[i] = a;
       }
     }
     __syncthreads();
   }
-  const float inv = 1.0f / l;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int i = 0; i < MAX_D / DA_WAVE; ++i) {
     const int d = lane + i * DA_WAVE;

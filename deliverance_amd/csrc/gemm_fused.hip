@@ -1,0 +1,211 @@
+// Decode-sized fused product: LayerNorm of the 32-bit residual rows, the bfloat16 product on the
+// matrix cores, bias / activation, and (for a q|k|v projection) the write of the new keys and
+// values into the paged cache -- one kernel where a step with a handful of rows would otherwise
+// pay for three.
+//
+//   a[m, :]   = LayerNorm(x[rows ? rows[m] : m, :]) rounded to bf16      (32-bit statistics)
+//   out[m, n] = act( sum_k a[m, k] * w[n, k] + bias[n] )
+//   columns n >= kv.q_cols of a q|k|v projection are also stored to the cache row kv.slot_map[m]
+//
+// Every block owns 16 output columns and all M <= 16*MT rows, and computes the statistics of
+// all rows itself (M * K floats from L2: cheap while M is small; the host uses the unfused
+// kernels for larger steps).  Statistics as in rowwise.hip: mean, then the centred sum of
+// squares, one wavefront per row, the row held in registers.
+// Formulas: core/src/main/java/io/teknek/deliverance/generator/LayerNorm.java:127-150,
+// CausalSelfAttention.java:266-291,315-336, MLPBlock.java:250-292.
+#include "gemm_common.h"
+
+#define FZ_COLS 16
+#define FZ_UNROLL 4
+#define FZ_VPL 8          // float4 per lane when a row is held in registers: K <= 2048
+
+struct LnPrologue {
+  const float* x;
+  const int* rows;
+  const void* g;
+  int g_dtype;
+  const void* b;
+  int b_dtype;
+  float eps;
+};
+
+struct KvScatter {
+  void* cache;          // null: no scatter
+  const int* slot_map;
+  int q_cols, kv_cols;  // k occupies columns [q_cols, q_cols+kv_cols), v the next kv_cols
+  int Hkv, D, page;
+};
+
+__device__ __forceinline__ void load8_param(const void* p, int dtype, int i, float* o) {
+  if (dtype == DA_BF16) {
+    const uint4 u = *(const uint4*)((const bf16_t*)p + i);
+    const uint32_t v[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o[2 * e] = __uint_as_float(v[e] << 16);
+      o[2 * e + 1] = __uint_as_float(v[e] & 0xffff0000u);
+    }
+  } else {
+    const float4 a = *(const float4*)((const float*)p + i), c = *(const float4*)((const float*)p + i + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = c.x; o[5] = c.y; o[6] = c.z; o[7] = c.w;
+  }
+}
+
+template <int MT, int NW>
+__global__ void __launch_bounds__(NW * 64)
+gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
+                      int M, int N, int K) {
+  __shared__ float red[NW][MT * 16][FZ_COLS + 1];
+  __shared__ float s_mean[MT * 16], s_rstd[MT * 16];
+  const int t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int n0 = blockIdx.x * FZ_COLS;
+  const int fr = lane % 16, fk = (lane / 16) * 8;
+
+  // ---- statistics of every row: wavefront v takes rows v, v + NW, ...
+  for (int m = wave; m < M; m += NW) {
+    const float* xr = ln.x + (size_t)(ln.rows ? ln.rows[m] : m) * K;
+    float4 v[FZ_VPL];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < FZ_VPL; ++i) {
+      const int c = (lane + i * 64) * 4;
+      v[i] = c < K ? *(const float4*)(xr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    const float mean = wave_sum(s) / (float)K;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < FZ_VPL; ++i) {
+      const int c = (lane + i * 64) * 4;
+      if (c < K) {
+        const float d0 = v[i].x - mean, d1 = v[i].y - mean, d2 = v[i].z - mean, d3 = v[i].w - mean;
+        q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)K + ln.eps);
+    if (lane == 0) { s_mean[m] = mean; s_rstd[m] = rstd; }
+  }
+  __syncthreads();
+
+  floatx4 acc[MT];
+  float mean[MT], rstd[MT];
+  bool arow_ok[MT];
+  const float* xp[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int m = i * 16 + fr;
+    arow_ok[i] = m < M;
+    const int ms = arow_ok[i] ? m : 0;
+    mean[i] = s_mean[ms]; rstd[i] = s_rstd[ms];
+    xp[i] = ln.x + (size_t)(ln.rows ? ln.rows[ms] : ms) * K + fk;
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const bool wrow_ok = n0 + fr < N;
+  const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
+
+  for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * FZ_UNROLL) {
+    uint4 wv[FZ_UNROLL];
+    float4 xa[FZ_UNROLL][MT][2];
+    float gg[FZ_UNROLL][8], bb[FZ_UNROLL][8];
+#pragma unroll
+    for (int u = 0; u < FZ_UNROLL; ++u) {
+      const int k = k0 + u * NW * 32;
+      const bool kin = k + fk < K;
+      const int ks = kin ? k : -fk;
+      wv[u] = load16(wp + ks);
+      if (!(kin && wrow_ok)) wv[u] = zero;
+      load8_param(ln.g, ln.g_dtype, ks + fk, gg[u]);
+      if (ln.b) load8_param(ln.b, ln.b_dtype, ks + fk, bb[u]);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        xa[u][i][0] = *(const float4*)(xp[i] + ks);
+        xa[u][i][1] = *(const float4*)(xp[i] + ks + 4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < FZ_UNROLL; ++u) {
+      const int k = k0 + u * NW * 32;
+      const bool kin = k + fk < K;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const float xs[8] = {xa[u][i][0].x, xa[u][i][0].y, xa[u][i][0].z, xa[u][i][0].w,
+                             xa[u][i][1].x, xa[u][i][1].y, xa[u][i][1].z, xa[u][i][1].w};
+        uint32_t pk[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float y0 = (xs[2 * e] - mean[i]) * rstd[i] * gg[u][2 * e];
+          float y1 = (xs[2 * e + 1] - mean[i]) * rstd[i] * gg[u][2 * e + 1];
+          if (ln.b) { y0 += bb[u][2 * e]; y1 += bb[u][2 * e + 1]; }
+          pk[e] = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
+        }
+        uint4 av = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        if (!(kin && arow_ok[i])) av = zero;
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                         __builtin_bit_cast(bf16x8_t, wv[u]), acc[i], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
+  __syncthreads();
+  for (int e = t; e < MT * 16 * FZ_COLS; e += NW * 64) {
+    const int m = e / FZ_COLS, c = e % FZ_COLS, n = n0 + c;
+    if (m < M && n < N) {
+      float v = red[0][m][c];
+#pragma unroll
+      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][m][c];
+      const float bias = ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
+      epilogue_store(ep, m, n, v, bias);
+      if (kv.cache && n >= kv.q_cols) {
+        const int slot = kv.slot_map[m];
+        if (slot >= 0) {
+          const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
+          const int h = cc / kv.D, d = cc % kv.D, pg = slot / kv.page, row = slot % kv.page;
+          const bf16_t val = f32_to_bf16(apply_act(v + bias, ep.act));
+          bf16_t* cache = (bf16_t*)kv.cache;
+          if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = val;
+          else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = val;
+        }
+      }
+    }
+  }
+}
+
+template <int NW>
+static void launch_fused(int mt, dim3 grid, hipStream_t s, const LnPrologue& ln, const bf16_t* W, int ldw,
+                         const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
+  if (mt == 1) hipLaunchKernelGGL((gemm_ln_skinny_kernel<1, NW>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_ln_skinny_kernel<2, NW>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
+}
+
+extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, int g_dtype, const void* b,
+                               int b_dtype, float eps, const void* w, int ldw, const void* bias, int bias_dtype,
+                               int act, void* out, int out_dtype, int ldo, int M, int N, int K, void* kv_cache,
+                               const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
+                               void* stream) {
+  DA_REQUIRE(M > 0 && M <= 32 && N > 0 && K > 0, "gemm_bf16_ln: takes 1..32 rows (M=%d N=%d K=%d)", M, N, K);
+  DA_REQUIRE(K % 8 == 0 && K <= 256 * FZ_VPL && ldw % 8 == 0 && ldw >= K && ldo >= N,
+             "gemm_bf16_ln: K must be a multiple of 8 up to %d (K=%d ldw=%d)", 256 * FZ_VPL, K, ldw);
+  DA_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
+             (!b || (uintptr_t)b % 16 == 0), "gemm_bf16_ln: operands must be 16-byte aligned");
+  DA_REQUIRE(eps > 0.f, "gemm_bf16_ln: eps must be > 0");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16_ln: unknown activation %d", act);
+  if (kv_cache) {
+    DA_REQUIRE(out_dtype == DA_BF16 && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N && page > 0,
+               "gemm_bf16_ln: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);
+  }
+  LnPrologue ln{x, rows, g, g_dtype, b, b_dtype, eps};
+  Epilogue ep{bias, bias_dtype, act, 0, out, out_dtype, ldo};
+  KvScatter kv{kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page};
+  dim3 grid(da_ceil_div(N, FZ_COLS));
+  const int mt = da_ceil_div(M, 16);
+  hipStream_t s = (hipStream_t)stream;
+  if (K >= 2048) launch_fused<16>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  else if (K >= 1024) launch_fused<8>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  else launch_fused<4>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  DA_CHECK_LAUNCH("gemm_bf16_ln");
+  return 0;
+}

@@ -7,8 +7,8 @@
 //
 //  * gemm_tile: 128x128 block tile, 4 wavefronts of 64x64 (2x2 MFMA 32x32x16), operands staged
 //    through LDS with a register prefetch of the next K-slab.  For steps with many rows (prefill).
-//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its 4
-//    wavefronts split K, stream their part of w straight from memory into MFMA 16x16x32
+//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its
+//    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
 //    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
 //
 // In both, an output element sums over k in an order that depends on K only, never on M or on
@@ -18,36 +18,13 @@
 // 8 consecutive k starting at 8 * (l / 32); it receives, for r in 0..15, the element at
 // row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
 // l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
-#include "common.h"
-
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+#include "gemm_common.h"
+#include <stdlib.h>
 
 #define BM 128
 #define BN 128
 #define BKT 64               // k per slab
 #define LDS_LD (BKT + 8)     // padded row length in elements (144 bytes): spreads rows over banks
-
-struct Epilogue {
-  const void* bias;
-  int bias_dtype;
-  int act;
-  int accumulate;
-  void* out;
-  int out_dtype;
-  int ldo;
-};
-
-__device__ __forceinline__ void epilogue_store(const Epilogue& ep, int m, int n, float v, float bias) {
-  v = apply_act(v + bias, ep.act);
-  const size_t o = (size_t)m * ep.ldo + n;
-  if (ep.accumulate) ((float*)ep.out)[o] += v;
-  else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
-  else ((float*)ep.out)[o] = v;
-}
-
-__device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }
 
 // ---------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
@@ -141,15 +118,16 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
-// M <= 64.  Block: 16 columns of the output, all rows; wavefront v takes the k-chunks
-// v, v+4, v+8, ... of 32 elements each.
+// M <= 64.  Block: 16 columns of the output, all rows; wavefront v of NW takes the k-chunks
+// v, v+NW, v+2NW, ... of 32 elements each, several of them in flight at a time.  NW grows with K
+// (fixed by K alone), so that the chain of dependent loads stays short.
 // ---------------------------------------------------------------------------------------------
 #define SK_COLS 16
-template <int MT>   // row tiles of 16
-__global__ void __launch_bounds__(256)
+template <int MT, int NW, int SK_UNROLL>   // row tiles of 16, wavefronts, k-chunks in flight per wavefront
+__global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                    Epilogue ep, int M, int N, int K) {
-  __shared__ float red[4][MT * 16][SK_COLS + 1];
+  __shared__ float red[NW][MT * 16][SK_COLS + 1];
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int n0 = blockIdx.x * SK_COLS;
   const int fr = lane % 16, fk = (lane / 16) * 8;
@@ -158,30 +136,60 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   const uint4 zero = make_uint4(0, 0, 0, 0);
   const bool wrow_ok = n0 + fr < N;
-  const bf16_t* wp = w + (size_t)(n0 + fr) * ldw + fk;
-  for (int k0 = wave * 32; k0 < K; k0 += 4 * 32) {
-    const bool kin = k0 + fk < K;
-    const uint4 wv = (wrow_ok && kin) ? load16(wp + k0) : zero;
-    const bf16x8_t bfrag = __builtin_bit_cast(bf16x8_t, wv);
+  const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
+  bool arow_ok[MT];
+  const bf16_t* ap[MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int m = i * 16 + fr;
-      const uint4 av = (m < M && kin) ? load16(a + (size_t)m * lda + k0 + fk) : zero;
-      acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), bfrag, acc[i], 0, 0, 0);
+  for (int i = 0; i < MT; ++i) {
+    arow_ok[i] = i * 16 + fr < M;
+    ap[i] = a + (size_t)(arow_ok[i] ? i * 16 + fr : 0) * lda + fk;
+  }
+  for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * SK_UNROLL) {
+    uint4 wv[SK_UNROLL], av[SK_UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u) {
+      const int k = k0 + u * NW * 32;
+      const bool kin = k + fk < K;
+      const int ks = kin ? k : -fk;             // a load that is not wanted reads the row's first chunk and is dropped
+      wv[u] = load16(wp + ks);
+      if (!(kin && wrow_ok)) wv[u] = zero;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        av[u][i] = load16(ap[i] + ks);
+        if (!(kin && arow_ok[i])) av[u][i] = zero;
+      }
     }
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u][i]),
+                                                         __builtin_bit_cast(bf16x8_t, wv[u]), acc[i], 0, 0, 0);
   }
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
   __syncthreads();
-  for (int e = t; e < MT * 16 * SK_COLS; e += 256) {
+  for (int e = t; e < MT * 16 * SK_COLS; e += NW * 64) {
     const int m = e / SK_COLS, c = e % SK_COLS, n = n0 + c;
     if (m < M && n < N) {
-      const float v = ((red[0][m][c] + red[1][m][c]) + red[2][m][c]) + red[3][m][c];
+      float v = red[0][m][c];
+#pragma unroll
+      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][m][c];
       epilogue_store(ep, m, n, v, ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f);
     }
   }
+}
+
+template <int NW>
+static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
+                          const Epilogue& ep, int M, int N, int K) {
+  // few rows leave registers for more chunks in flight
+  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
+  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
+  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
 }
 
 extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
@@ -202,10 +210,15 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   if (M <= 64) {
     dim3 grid(da_ceil_div(N, SK_COLS));
     const int mt = da_ceil_div(M, 16);
-    if (mt == 1) hipLaunchKernelGGL(gemm_skinny_kernel<1>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
-    else if (mt == 2) hipLaunchKernelGGL(gemm_skinny_kernel<2>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
-    else if (mt == 3) hipLaunchKernelGGL(gemm_skinny_kernel<3>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
-    else hipLaunchKernelGGL(gemm_skinny_kernel<4>, grid, dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K);
+    // the number of wavefronts that split K depends on K alone, so a row's sums keep their order
+    static int force_nw = -1;
+    if (force_nw < 0) { const char* e = getenv("DA_SKINNY_NW"); force_nw = e ? atoi(e) : 0; }
+    int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
+    if (force_nw > 0) nw = force_nw;
+    if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
+    else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
+    else if (nw == 4) launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
+    else launch_skinny<2>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
   } else {
     const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
     hipLaunchKernelGGL(gemm_tile_kernel, dim3(tiles_m * tiles_n), dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K,

@@ -73,15 +73,89 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
   }
 }
 
+__device__ __forceinline__ float4 load_param4(const void* p, int dtype, int i) {
+  if (dtype == DA_BF16) {
+    const uint2 u = *(const uint2*)((const bf16_t*)p + i);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+  }
+  return *(const float4*)((const float*)p + i);
+}
+
+// The same norm with the whole row held in registers: every load of the row is in flight at
+// once, which is what counts when a step has a handful of rows.  E a multiple of 4, E <= 256*VPL.
+template <int VPL>
+__global__ void __launch_bounds__(DA_WAVE)
+layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                     const void* __restrict__ w, int w_dtype, const void* __restrict__ b, int b_dtype,
+                     float eps, void* __restrict__ y, int y_dtype, int E) {
+  const int lane = threadIdx.x, r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * E;
+  float4 v[VPL];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int c = (lane + i * DA_WAVE) * 4;
+    v[i] = c < E ? *(const float4*)(xr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+  }
+  const float mean = wave_sum(s) / (float)E;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int c = (lane + i * DA_WAVE) * 4;
+    if (c < E) {
+      const float d0 = v[i].x - mean, d1 = v[i].y - mean, d2 = v[i].z - mean, d3 = v[i].w - mean;
+      q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    }
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(q) / (float)E + eps);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int c = (lane + i * DA_WAVE) * 4;
+    if (c < E) {
+      const float4 g = load_param4(w, w_dtype, c);
+      float4 o = make_float4((v[i].x - mean) * inv * g.x, (v[i].y - mean) * inv * g.y,
+                             (v[i].z - mean) * inv * g.z, (v[i].w - mean) * inv * g.w);
+      if (b) {
+        const float4 bb = load_param4(b, b_dtype, c);
+        o.x += bb.x; o.y += bb.y; o.z += bb.z; o.w += bb.w;
+      }
+      if (y_dtype == DA_BF16) {
+        uint2 u;
+        u.x = (uint32_t)f32_to_bf16(o.x) | ((uint32_t)f32_to_bf16(o.y) << 16);
+        u.y = (uint32_t)f32_to_bf16(o.z) | ((uint32_t)f32_to_bf16(o.w) << 16);
+        *(uint2*)((bf16_t*)y + (size_t)r * E + c) = u;
+      } else {
+        *(float4*)((float*)y + (size_t)r * E + c) = o;
+      }
+    }
+  }
+}
+
 extern "C" int da_layernorm(const float* x, const int* rows, const void* w, int w_dtype,
                             const void* b, int b_dtype, float eps, void* y, int y_dtype, int R,
                             int E, void* stream) {
   DA_REQUIRE(R >= 0 && E > 0, "layernorm: bad sizes R=%d E=%d", R, E);
   DA_REQUIRE(eps > 0.f, "layernorm: eps must be > 0");
   if (R == 0) return 0;
-  const int waves = 4;
-  hipLaunchKernelGGL(layernorm_kernel, dim3(da_ceil_div(R, waves)), dim3(waves * DA_WAVE), 0,
-                     (hipStream_t)stream, x, rows, w, w_dtype, b, b_dtype, eps, y, y_dtype, R, E);
+  hipStream_t st = (hipStream_t)stream;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                       (!b || (uintptr_t)b % 16 == 0);
+  if (E % 4 == 0 && E <= 2048 && aligned) {
+#define LN_LAUNCH(V)                                                                                      \
+  hipLaunchKernelGGL(layernorm_row_kernel<V>, dim3(R), dim3(DA_WAVE), 0, st, x, rows, w, w_dtype, b, b_dtype, \
+                     eps, y, y_dtype, E)
+    if (E <= 256) LN_LAUNCH(1);
+    else if (E <= 512) LN_LAUNCH(2);
+    else if (E <= 1024) LN_LAUNCH(4);
+    else LN_LAUNCH(8);
+#undef LN_LAUNCH
+  } else {
+    const int waves = 4;
+    hipLaunchKernelGGL(layernorm_kernel, dim3(da_ceil_div(R, waves)), dim3(waves * DA_WAVE), 0, st, x, rows, w,
+                       w_dtype, b, b_dtype, eps, y, y_dtype, R, E);
+  }
   DA_CHECK_LAUNCH("layernorm");
   return 0;
 }

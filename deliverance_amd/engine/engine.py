@@ -64,7 +64,8 @@ class CausalLanguageModel:
             tokens = max(tokens, engine_config.page_size)
         n_slots = engine_config.state_slots if engine_config.state_slots is not None else engine_config.max_num_seqs
         self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots)
-        self.runner = StepRunner(model, self.cache)
+        self.runner = StepRunner(model, self.cache, use_graphs=engine_config.use_graphs,
+                                 max_graph_batch=max(engine_config.max_num_seqs, 1))
         self.scheduler = Scheduler(self.cache.manager, model.config.max_positions, model.config.eos_token_ids,
                                    engine_config.max_num_seqs, engine_config.max_batch_tokens,
                                    engine_config.max_chunk, on_open=self.cache.reset_state)
@@ -107,14 +108,16 @@ class CausalLanguageModel:
             if s.samples:
                 records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))
                 samplers.append(s)
-        logits, ctx = self.runner.run(entries, reserved=True, extra_words=records or None)
+        logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
         sampled: Dict[Hashable, int] = {}
         if samplers:
             R = len(samplers)
             if self._sampled_dev.numel() < R:
                 self._sampled_dev = torch.empty(2 * R, dtype=torch.int32, device=self.model.device)
-            out = self._sampled_dev[:R]
-            ops.sample(logits, ctx.extra, out)
+            out = getattr(ctx, "sampled", None)       # a replayed graph has sampled already
+            if out is None:
+                out = self._sampled_dev[:R]
+                ops.sample(logits, ctx.extra, out)
             want_lp = [s for s in samplers if s.request.params.log_probs and s.request.params.top_log_probs > 0]
             lp = None
             if want_lp:

@@ -33,7 +33,7 @@ class StepError(ValueError):
 
 
 class StepRunner:
-    def __init__(self, model: CausalLM, cache: DeviceCache):
+    def __init__(self, model: CausalLM, cache: DeviceCache, use_graphs: bool = False, max_graph_batch: int = 256):
         self.model = model
         self.cache = cache
         self.device = model.device
@@ -43,6 +43,9 @@ class StepRunner:
         self._copied = None
         self.max_blocks_cap = -(-model.config.max_positions // cache.page_size)
         self.last_ctx: Optional[StepContext] = None
+        self.use_graphs = use_graphs
+        self.max_graph_batch = max_graph_batch
+        self._graphs = {}
 
     # ---- host -> device in one copy --------------------------------------------------------
     def _upload(self, words: List[int]) -> torch.Tensor:
@@ -62,11 +65,14 @@ class StepRunner:
 
     # ---- the step --------------------------------------------------------------------------
     def run(self, entries: Sequence[StepEntry], reserved: bool = False,
-            extra_words: Optional[List[int]] = None):
+            sample_records: Optional[List[int]] = None):
         """Run one step.  Returns (logits [R, V] float32 on the device, ctx).  The rows follow
         the order of ``entries`` and of each entry's ``want``.  With ``reserved`` the caller has
         already opened the requests and reserved their positions (``CacheManager.extend``).
-        ``extra_words`` ride along in the same host-to-device copy (``ctx.extra``)."""
+        ``sample_records`` (8 words per wanted row, see sampling.device_record) ride along in the
+        same host-to-device copy (``ctx.extra``); when they are given and the step holds one-token
+        sequences only, the step and its sampling are replayed from a recorded HIP graph and the
+        sampled tokens are left in ``ctx.sampled``."""
         mgr = self.cache.manager
         cfg = self.model.config
         if not entries:
@@ -112,7 +118,35 @@ class StepRunner:
         # one-token entries first (the decode kernels take them), portions after
         order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
         n_decode = sum(1 for e in entries if len(e.tokens) == 1)
-        S = len(entries)
+        graph_ok = (sample_records is not None and n_decode == len(entries) and self.use_graphs
+                    and len(entries) <= self.max_graph_batch and all(list(e.want) == [0] for e in entries))
+        if graph_ok:
+            logits, ctx = self._run_graph(entries, starts, sample_records)
+            if not reserved:
+                for e in entries:
+                    mgr.commit(e.rid)
+            return logits, ctx
+
+        words, offs, meta = self._pack(entries, order, starts, pad_to=None, max_blocks=None,
+                                       extra=sample_records)
+        dev = self._upload(words)
+        ctx = self._context(dev, offs, meta, self.arena)
+        self.last_ctx = ctx
+        R = meta["R"]
+        logits = self.model.forward(ctx, ctx.want_rows if R else None, R)
+        if not reserved:                 # who reserves commits: the scheduler does it for its batches
+            for e in entries:
+                mgr.commit(e.rid)
+        return logits, ctx
+
+    # ---- packing the step's integers -----------------------------------------------------------
+    def _pack(self, entries, order, starts, pad_to, max_blocks, extra):
+        """All integers of a step in one list: tokens, positions, sequence ids, row starts, lengths,
+        state slots, wanted rows, then per cache group the cache row of every token and the block
+        tables, then ``extra``.  With ``pad_to`` the step is filled up with empty one-token
+        sequences (length 0, no cache row), so that its shape is fixed."""
+        mgr = self.cache.manager
+        S_real = len(entries)
         tokens: List[int] = []
         positions: List[int] = []
         seq_of: List[int] = []
@@ -130,12 +164,16 @@ class StepRunner:
             q_start.append(len(tokens))
             seq_lens.append(st + len(e.tokens))
             state_slots.append(mgr.state_slot(e.rid))
-        N = len(tokens)
         want_rows = [row0[i] + int(w) for i, e in enumerate(entries) for w in e.want]
-        R = len(want_rows)
-
+        n_pad = 0 if pad_to is None else pad_to - S_real
+        for k in range(n_pad):
+            tokens.append(0); positions.append(0); seq_of.append(S_real + k)
+            q_start.append(len(tokens)); seq_lens.append(0); state_slots.append(-1)
+            want_rows.append(len(tokens) - 1)
+        N, S, R = len(tokens), S_real + n_pad, len(want_rows)
         G = len(self.cache.groups)
-        max_blocks = max(1, max(len(mgr.table(entries[i].rid, g)) for i in order for g in range(G))) if G else 1
+        if max_blocks is None:
+            max_blocks = max(1, max(len(mgr.table(entries[i].rid, g)) for i in order for g in range(G))) if G else 1
         words = tokens + positions + seq_of + q_start + seq_lens + state_slots + want_rows
         offs = {}
         o = 0
@@ -151,37 +189,86 @@ class StepRunner:
                 sm += mgr.slots_for(e.rid, g, starts[e.rid], len(e.tokens))
                 t = mgr.table(e.rid, g)
                 bt += t + [-1] * (max_blocks - len(t))
+            sm += [-1] * n_pad
+            bt += [-1] * (n_pad * max_blocks)
             words += sm + bt
             offs[f"slot_map{g}"] = (o, N)
             offs[f"block_table{g}"] = (o + N, S * max_blocks)
             o += N + S * max_blocks
-        if extra_words:
-            words += extra_words
-            offs["extra"] = (o, len(extra_words))
-        dev = self._upload(words)
+        if extra:
+            extra = list(extra) + [0] * (8 * n_pad if pad_to is not None else 0)
+            words += extra
+            offs["extra"] = (o, len(extra))
+        meta = dict(N=N, S=S, R=R, G=G, max_blocks=max_blocks, n_decode=sum(1 for e in entries if len(e.tokens) == 1) + n_pad,
+                    q_start=q_start, seq_lens=seq_lens, state_slots=state_slots)
+        return words, offs, meta
 
+    def _context(self, dev, offs, meta, arena) -> StepContext:
         def view(name):
             a, n = offs[name]
             return dev[a:a + n]
-
+        N, S, G, max_blocks = meta["N"], meta["S"], meta["G"], meta["max_blocks"]
         ctx = StepContext()
         ctx.device = self.device
         ctx.dtype = self.model.dtype
-        ctx.n_tokens, ctx.n_seqs, ctx.n_decode = N, S, n_decode
+        ctx.n_tokens, ctx.n_seqs, ctx.n_decode = N, S, meta["n_decode"]
         ctx.tokens, ctx.positions, ctx.seq_of_token = view("tokens"), view("positions"), view("seq_of")
         ctx.q_start, ctx.seq_lens, ctx.state_slots = view("q_start"), view("seq_lens"), view("state_slots")
-        ctx.q_start_host, ctx.seq_lens_host, ctx.state_slots_host = q_start, seq_lens, state_slots
-        ctx.max_query_len = max(q_start[s + 1] - q_start[s] for s in range(S))
-        ctx.max_seq_len = max(seq_lens)
+        ctx.q_start_host, ctx.seq_lens_host, ctx.state_slots_host = meta["q_start"], meta["seq_lens"], meta["state_slots"]
+        ctx.max_query_len = max(meta["q_start"][s + 1] - meta["q_start"][s] for s in range(S))
+        ctx.max_seq_len = max(meta["seq_lens"])
         ctx.block_tables = [view(f"block_table{g}").view(S, max_blocks) for g in range(G)]
         ctx.slot_maps = [view(f"slot_map{g}") for g in range(G)]
         ctx.cache = self.cache
-        ctx._arena = self.arena
-        ctx.extra = view("extra") if extra_words else None
+        ctx._arena = arena
+        ctx.extra = view("extra") if "extra" in offs else None
+        ctx.want_rows = view("want")
+        return ctx
+
+    # ---- decode-only steps replayed from a HIP graph ----------------------------------------------
+    def _run_graph(self, entries, starts, sample_records):
+        """A step of one-token sequences only has a fixed shape once it is padded to a bucket
+        size, so its kernels (model and sampling) are recorded once per bucket and replayed.
+        Only the step's integers change: they are copied into the bucket's own buffer first."""
+        from ..kernels import ops
+        S = len(entries)
+        bucket = 1
+        while bucket < S:
+            bucket *= 2
+        order = list(range(S))
+        words, offs, meta = self._pack(entries, order, starts, pad_to=bucket, max_blocks=self.max_blocks_cap,
+                                       extra=sample_records)
+        st = self._graphs.get(bucket)
+        if st is None:
+            st = {"dev": torch.empty(len(words), dtype=torch.int32, device=self.device),
+                  "host": torch.empty(len(words), dtype=torch.int32, pin_memory=True),
+                  "arena": Arena(self.device), "graph": None, "copied": None,
+                  "tokens": torch.empty(bucket, dtype=torch.int32, device=self.device)}
+            self._graphs[bucket] = st
+        assert st["dev"].numel() == len(words), "a bucket's layout is fixed"
+        if st["copied"] is not None:
+            st["copied"].synchronize()
+        st["host"].copy_(torch.tensor(words, dtype=torch.int32))
+        st["dev"].copy_(st["host"], non_blocking=True)
+        st["copied"] = torch.cuda.Event()
+        st["copied"].record()
+        ctx = self._context(st["dev"], offs, meta, st["arena"])
         self.last_ctx = ctx
 
-        logits = self.model.forward(ctx, view("want") if R else None, R)
-        if not reserved:                 # who reserves commits: the scheduler does it for its batches
-            for e in entries:
-                mgr.commit(e.rid)
-        return logits, ctx
+        def body():
+            logits = self.model.forward(ctx, ctx.want_rows, bucket)
+            ops.sample(logits, ctx.extra, st["tokens"])
+            return logits
+
+        if st["graph"] is None:
+            st["logits"] = body()                      # eager once: sizes the bucket's scratch buffers
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                st["logits"] = body()
+            st["graph"] = g
+            # the eager run above already did this step's work; the recorded graph is used from the next step on
+        else:
+            st["graph"].replay()
+        ctx.sampled = st["tokens"][:S]
+        return st["logits"][:S], ctx

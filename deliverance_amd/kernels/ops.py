@@ -222,6 +222,55 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     return out
 
 
+FUSED_LN_MAX_ROWS = 32
+FUSED_LN_MAX_K = 2048
+
+
+def can_fuse_ln(n_rows: int, x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``linear_ln`` takes this step: few rows, bfloat16 weights, a width the kernel holds."""
+    K = w.shape[1]
+    return (_MODE == "tuned" and w.dtype == torch.bfloat16 and 0 < n_rows <= FUSED_LN_MAX_ROWS
+            and K % 8 == 0 and K <= FUSED_LN_MAX_K and w.stride(0) % 8 == 0 and x.dtype == torch.float32)
+
+
+def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_weight: torch.Tensor,
+              norm_bias: Optional[torch.Tensor], eps: float, w: torch.Tensor, bias: Optional[torch.Tensor],
+              out: torch.Tensor, act: Optional[str] = None, kv_cache: Optional[torch.Tensor] = None,
+              slot_map: Optional[torch.Tensor] = None, q_cols: int = 0) -> torch.Tensor:
+    """out = act(LayerNorm(x[rows]) @ w.T + bias) in one kernel, for steps of at most 32 rows; with
+    ``kv_cache`` the columns from ``q_cols`` on (k | v of a fused projection) also go to the cache
+    rows ``slot_map``."""
+    _dev(x, rows, norm_weight, norm_bias, w, bias, out, kv_cache, slot_map)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "linear_ln: x must be contiguous float32")
+    _rows_2d(w, "w"); _rows_2d(out, "out")
+    N, K = w.shape
+    _need(x.shape[1] == K and norm_weight.numel() == K and (norm_bias is None or norm_bias.numel() == K),
+          "linear_ln: widths differ")
+    _need(w.dtype == torch.bfloat16, "linear_ln: w must be bfloat16")
+    _need(0 < n_rows <= FUSED_LN_MAX_ROWS and out.shape[0] >= n_rows and out.shape[1] == N, "linear_ln: bad row count")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "linear_ln: fewer rows in x than asked")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "linear_ln: rows must be int32")
+    _need(bias is None or bias.numel() == N, "linear_ln: bias length differs from N")
+    _need(act in ACTIVATIONS, f"linear_ln: unknown activation {act!r}")
+    Hkv = D = page = kv_cols = 0
+    if kv_cache is not None:
+        _need(kv_cache.dim() == 5 and kv_cache.is_contiguous() and kv_cache.dtype == torch.bfloat16 and
+              out.dtype == torch.bfloat16, "linear_ln: cache slot must be contiguous bfloat16 [pages,2,Hkv,page,D]")
+        _, _, Hkv, page, D = kv_cache.shape
+        kv_cols = Hkv * D
+        _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
+              "linear_ln: slot_map must be int32 [rows]")
+        _need(q_cols + 2 * kv_cols == N, "linear_ln: q|k|v columns do not add up to N")
+    _check(build.load().da_gemm_bf16_ln(
+        _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), _ptr(norm_bias),
+        _dt(norm_bias) if norm_bias is not None else 0, ctypes.c_float(eps), _ptr(w), w.stride(0), _ptr(bias),
+        _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0), n_rows, N, K,
+        _ptr(kv_cache), _ptr(slot_map), q_cols, kv_cols, Hkv, D, page, _stream()))
+    return out
+
+
 def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)

@@ -77,6 +77,10 @@ class CausalLM:
         logits = ctx.buf("logits", n_want, self.config.vocab_size, torch.float32)
         if n_want == 0:
             return logits
+        from ..parts.norms import LayerNorm
+        if isinstance(self.final_norm, LayerNorm) and ops.can_fuse_ln(n_want, x, self.head_weight):
+            fn = self.final_norm                   # few wanted rows: norm and head in one kernel
+            return ops.linear_ln(x, want_rows, n_want, fn.weight, fn.bias, fn.eps, self.head_weight, None, logits)
         if self.final_norm is not None:
             e = self.final_norm.forward(ctx, x, rows=want_rows, n_rows=n_want, out_name="final_norm")
         else:

@@ -43,6 +43,22 @@ class CausalSelfAttention(Mixer):
     def cache_need(self):
         return KVNeed(self.n_kv_heads, self.head_dim, self.window)
 
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call) -> bool:
+        """Small steps: LayerNorm, the q|k|v projection and the cache write in one kernel."""
+        from .norms import LayerNorm
+        N = x.shape[0]
+        if not (isinstance(norm, LayerNorm) and self.position is None
+                and ops.can_fuse_ln(N, x, self.qkv_weight)):
+            return False
+        qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
+        slot = ctx.cache.kv[call.cache]
+        group = ctx.group_of(call.cache)
+        ops.linear_ln(x, None, N, norm.weight, norm.bias, norm.eps, self.qkv_weight, self.qkv_bias, qkv,
+                      kv_cache=slot if call.write else None, slot_map=ctx.slot_maps[group] if call.write else None,
+                      q_cols=self.q_cols)
+        self._attend(ctx, qkv, x, slot, group)
+        return True
+
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
         N = h.shape[0]
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
@@ -54,6 +70,10 @@ class CausalSelfAttention(Mixer):
         if call.write:
             ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
                          self.n_kv_heads, self.head_dim)
+        self._attend(ctx, qkv, x, slot, group)
+
+    def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int) -> None:
+        N = qkv.shape[0]
         o = ctx.buf("attn_out", N, self.q_cols, ctx.dtype)
         ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
         ops.linear(o, self.out_weight, self.out_bias, x, accumulate=True)

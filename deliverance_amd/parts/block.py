@@ -26,15 +26,21 @@ class Block:
             # needs the part to write to a buffer of its own instead of into the stream.
             raise NotImplementedError("post-part norms are not wired yet")
 
-    def _sub(self, ctx, x, pre, run):
+    @staticmethod
+    def _normed(ctx, x, pre):
         if pre is not None:
-            h = pre.forward(ctx, x)
-        else:
-            h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)
-            h.copy_(x)
-        run(h)
+            return pre.forward(ctx, x)
+        h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)
+        h.copy_(x)
+        return h
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
-        self._sub(ctx, x, self.pre_mixer_norm, lambda h: self.mixer.forward(ctx, h, x, call))
+        # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm itself
+        # (fused into its first product) and returns True, or returns False to decline this step.
+        fused = getattr(self.mixer, "forward_normed", None)
+        if not (fused is not None and self.pre_mixer_norm is not None and fused(ctx, self.pre_mixer_norm, x, call)):
+            self.mixer.forward(ctx, self._normed(ctx, x, self.pre_mixer_norm), x, call)
         if self.feed_forward is not None:
-            self._sub(ctx, x, self.pre_ff_norm, lambda h: self.feed_forward.forward(ctx, h, x))
+            fused = getattr(self.feed_forward, "forward_normed", None)
+            if not (fused is not None and self.pre_ff_norm is not None and fused(ctx, self.pre_ff_norm, x)):
+                self.feed_forward.forward(ctx, self._normed(ctx, x, self.pre_ff_norm), x)

@@ -23,6 +23,18 @@ class DenseFeedForward(FeedForward):
         if tuple(self.proj_weight.shape) != (self.width, self.inner):
             raise ValueError(f"proj weight is {list(self.proj_weight.shape)}, expected {[self.width, self.inner]}")
 
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor) -> bool:
+        """Small steps: LayerNorm, fc, bias and activation in one kernel."""
+        from .norms import LayerNorm
+        N = x.shape[0]
+        if not (isinstance(norm, LayerNorm) and ops.can_fuse_ln(N, x, self.fc_weight)):
+            return False
+        mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)
+        ops.linear_ln(x, None, N, norm.weight, norm.bias, norm.eps, self.fc_weight, self.fc_bias, mid,
+                      act=self.activation)
+        ops.linear(mid, self.proj_weight, self.proj_bias, x, accumulate=True)
+        return True
+
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
         N = h.shape[0]
         mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)

@@ -360,3 +360,41 @@ def test_xtc_and_logprobs(ops):
     top = torch.topk(want, 4)
     assert idx[0].cpu().tolist() == top.indices.tolist()
     assert (lp[0].cpu().double() - top.values).abs().max() < 1e-4
+
+
+# ----------------------------------------------------------------------------- fused norm + product
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 2304, 768), (17, 1000, 96), (32, 200, 1600), (5, 50257, 768)])
+@pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
+def test_fused_norm_product(ops, M, N, K, pdtype):
+    g = torch.Generator().manual_seed(M + N)
+    x = (torch.randn(M + 3, K, generator=g) * 2 + 1).to(DEV)
+    gw, gb = torch.randn(K, generator=g).to(pdtype).to(DEV), torch.randn(K, generator=g).to(pdtype).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
+    bias = bf(torch.randn(N, generator=g)).to(DEV)
+    rows = torch.tensor([(i * 7) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
+    a = F.layer_norm(x.double(), (K,), gw.double(), gb.double(), 1e-5)[rows.long()].to(torch.bfloat16).double()
+    for act, od in ((None, torch.float32), ("gelu_new", torch.bfloat16)):
+        out = torch.empty(M, N, device=DEV, dtype=od)
+        ops.linear_ln(x, rows, M, gw, gb, 1e-5, w, bias, out, act=act)
+        ref = a @ w.double().t() + bias.double()
+        if act:
+            ref = F.gelu(ref, approximate="tanh")
+        tol = (2e-2 if od == torch.bfloat16 else 2e-3) * max(1.0, ref.abs().max().item())
+        assert (out.double() - ref).abs().max() < tol
+
+
+def test_fused_norm_product_writes_keys_and_values(ops):
+    g = torch.Generator().manual_seed(11)
+    Hq, Hkv, D, page, M, K = 6, 2, 48, 16, 9, 96
+    N = (Hq + 2 * Hkv) * D
+    x = torch.randn(M, K, generator=g).to(DEV)
+    gw, gb = bf(torch.randn(K, generator=g)).to(DEV), bf(torch.randn(K, generator=g)).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
+    bias = bf(torch.randn(N, generator=g)).to(DEV)
+    slots = torch.tensor([3 * page + 5, -1, 0, 17, 40, 41, 42, 95, 64], dtype=torch.int32, device=DEV)
+    c1 = torch.zeros(6, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
+    c2 = torch.zeros_like(c1)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops.linear_ln(x, None, M, gw, gb, 1e-5, w, bias, out, kv_cache=c1, slot_map=slots, q_cols=Hq * D)
+    ops.kv_write(out, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)      # the separate kernel on the same rows
+    assert torch.equal(c1, c2) and c1.abs().sum() > 0
