@@ -24,6 +24,7 @@ from ..config.engine_config import EngineConfig
 from ..kernels import ops
 from ..models.causal_lm import CausalLM, load_model
 from ..parts.base import KVNeed
+from ..profiler import InferenceProfiler
 from ..sampling.params import GeneratorParameters
 from ..sampling.sampler import RECORD_WORDS, device_record
 from .device_cache import DeviceCache
@@ -94,7 +95,8 @@ class CausalLanguageModel:
         """One scheduler decision, one model step, one sampling call.  Returns the requests
         that finished in this step."""
         before = len(self.scheduler.finished)
-        batch: List[Scheduled] = self.scheduler.schedule()
+        with InferenceProfiler.timer("scheduler.schedule"):
+            batch: List[Scheduled] = self.scheduler.schedule()
         failed = self.scheduler.finished[before:]
         if not batch:
             return list(failed)
@@ -108,7 +110,10 @@ class CausalLanguageModel:
             if s.samples:
                 records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))
                 samplers.append(s)
-        logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
+        decode_only = all(s.n == 1 for s in batch)
+        with InferenceProfiler.timer("generation.decode" if decode_only else "generation.prefill"):
+            logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
+        InferenceProfiler.counter("engine.batch_tokens", sum(s.n for s in batch))
         sampled: Dict[Hashable, int] = {}
         if samplers:
             R = len(samplers)
@@ -126,7 +131,8 @@ class CausalLanguageModel:
                 val = torch.empty((R, n), dtype=torch.float32, device=self.model.device)
                 ops.top_logprobs(logits, ctx.extra, n, idx, val)
                 lp = (idx.cpu(), val.cpu())
-            host = out.cpu()                                   # the step's one synchronisation
+            with InferenceProfiler.timer("sampler.sample"):
+                host = out.cpu()                               # the step's one synchronisation
             for i, s in enumerate(samplers):
                 sampled[s.request.rid] = int(host[i])
                 p = s.request.params

@@ -43,7 +43,7 @@ class StepRunner:
         self._copied = None
         self.max_blocks_cap = -(-model.config.max_positions // cache.page_size)
         self.last_ctx: Optional[StepContext] = None
-        self.use_graphs = use_graphs
+        self.use_graphs = use_graphs and model.graph_safe
         self.max_graph_batch = max_graph_batch
         self._graphs = {}
 

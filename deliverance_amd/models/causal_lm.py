@@ -45,6 +45,11 @@ class CausalLM:
             if not (0 <= call.layer < len(self.blocks)):
                 raise ValueError(f"run order names layer {call.layer}, the model has {len(self.blocks)}")
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether every part allows a decode step to be replayed from a recorded HIP graph."""
+        return all(b.mixer.graph_safe and (b.feed_forward is None or b.feed_forward.graph_safe) for b in self.blocks)
+
     # ---- what the cache must provide -----------------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
         """cache slot -> KVNeed / StateNeed of the layer call that writes it."""

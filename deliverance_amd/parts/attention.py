@@ -16,6 +16,8 @@ from .base import (KVNeed, Mixer, StepContext, build_position, register_mixer, t
 
 
 class CausalSelfAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec, params, dtype, device):
         self.spec = spec
         self.n_heads, self.n_kv_heads, self.head_dim = spec.n_heads, spec.n_kv_heads, spec.head_dim

@@ -68,7 +68,6 @@ class StepContext:
         self.slot_maps: List[torch.Tensor] = []        # per group int32 [N]
         self.cache = None                              # engine.DeviceCache
         self._arena = None
-        self.fixed_shapes = False                      # True while a HIP graph is recorded
 
     def buf(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         """A scratch matrix [rows, cols] that lives until the step ends."""
@@ -102,6 +101,11 @@ class Norm:
 
 
 class Mixer:
+    # True when `forward` launches the same kernels with the same arguments for every step of one
+    # shape and reads the step's data from device memory only: then a decode step can be recorded
+    # once as a HIP graph and replayed.  A mixer that reads ctx.*_host must leave this False.
+    graph_safe = False
+
     def cache_need(self):
         return None
 
@@ -110,6 +114,8 @@ class Mixer:
 
 
 class FeedForward:
+    graph_safe = False
+
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
         raise NotImplementedError
 

@@ -10,6 +10,8 @@ from .base import FeedForward, StepContext, register_feed_forward, to_matrix, to
 
 
 class DenseFeedForward(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, params, dtype, device):
         self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
         if self.activation not in ops.ACTIVATIONS:

@@ -1,0 +1,196 @@
+"""Each part alone (norm, positions, attention mixer, feed-forward, block) against the plain
+functions, built from its spec and parameters only, in 32-bit and in bfloat16."""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {torch.float32: 3e-5, torch.bfloat16: 4e-2}
+
+
+def make_ctx(dtype, lens_new, past, n_kv_heads, head_dim, page=16, n_slots=1, window=None):
+    """A step context by hand: sequences with `past` cached positions bring `lens_new` tokens."""
+    from deliverance_amd.parts import Arena, StepContext
+    S = len(lens_new)
+    order = sorted(range(S), key=lambda i: (lens_new[i] != 1, i))
+    lens_new = [lens_new[i] for i in order]
+    past = [past[i] for i in order]
+    total = [p + n for p, n in zip(past, lens_new)]
+    n_pages = sum(-(-t // page) for t in total) + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(1)).tolist()
+    max_blocks = max(-(-t // page) for t in total)
+    bt = torch.full((S, max_blocks), -1, dtype=torch.int32)
+    for s, t in enumerate(total):
+        for j in range(-(-t // page)):
+            bt[s, j] = perm.pop()
+    ctx = StepContext()
+    ctx.device, ctx.dtype = torch.device(DEV), dtype
+    ctx.n_seqs, ctx.n_tokens = S, sum(lens_new)
+    ctx.n_decode = sum(1 for n in lens_new if n == 1)
+    pos, seq_of, slots, q_start = [], [], [], [0]
+    for s in range(S):
+        for i in range(lens_new[s]):
+            p_ = past[s] + i
+            pos.append(p_); seq_of.append(s); slots.append(int(bt[s, p_ // page]) * page + p_ % page)
+        q_start.append(len(pos))
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ctx.positions, ctx.seq_of_token, ctx.q_start, ctx.seq_lens = dev(pos), dev(seq_of), dev(q_start), dev(total)
+    ctx.tokens = dev([0] * len(pos))
+    ctx.q_start_host, ctx.seq_lens_host = q_start, total
+    ctx.max_query_len, ctx.max_seq_len = max(lens_new), max(total)
+    ctx.block_tables, ctx.slot_maps = [bt.to(DEV)], [dev(slots)]
+    kv = {i: torch.full((n_pages, 2, n_kv_heads, page, head_dim), float("nan"), dtype=dtype, device=DEV) for i in range(n_slots)}
+    ctx.cache = SimpleNamespace(kv=kv, group_of_slot={i: 0 for i in range(n_slots)})
+    ctx._arena = Arena(DEV)
+    ctx.order = order
+    return ctx
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from deliverance_amd.config import NormSpec
+    from deliverance_amd.parts import build_norm
+    g = torch.Generator().manual_seed(0)
+    E = 200
+    w, b = torch.randn(E, generator=g).to(torch.bfloat16), torch.randn(E, generator=g).to(torch.bfloat16)
+    norm = build_norm(NormSpec("layernorm", E, 1e-6), {"weight": w, "bias": b}, dtype, DEV)
+    assert norm.weight.dtype == (torch.float32 if dtype == torch.float32 else torch.bfloat16)   # stored dtype kept in serving
+    ctx = make_ctx(dtype, [5], [0], 1, 16)
+    x = (torch.randn(5, E, generator=g) * 2).to(DEV)
+    got = norm.forward(ctx, x)
+    want = P.layer_norm(x.double().cpu().numpy(), w.double().numpy(), b.double().numpy(), 1e-6)
+    assert got.dtype == dtype and np.abs(got.double().cpu().numpy() - want).max() < TOL[dtype]
+    nobias = build_norm(NormSpec("layernorm", E, 1e-6, bias=False), {"weight": w}, dtype, DEV)
+    got = nobias.forward(ctx, x)
+    want = P.layer_norm(x.double().cpu().numpy(), w.double().numpy(), None, 1e-6)
+    assert np.abs(got.double().cpu().numpy() - want).max() < TOL[dtype]
+    with pytest.raises(KeyError, match="no norm of kind"):
+        build_norm(NormSpec("rmsnorm", E, 1e-6), {"weight": w}, dtype, DEV)
+
+
+def test_learned_positions_part():
+    from deliverance_amd.config import PositionSpec
+    from deliverance_amd.kernels import ops
+    from deliverance_amd.parts import build_position
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(40, 32, generator=g).to(torch.bfloat16)
+    pos = build_position(PositionSpec("learned", 40), {"table": table}, torch.bfloat16, DEV)
+    wte = torch.randn(100, 32, generator=g).to(torch.bfloat16).to(DEV)
+    ids = torch.tensor([3, 99, 0], dtype=torch.int32, device=DEV)
+    where = torch.tensor([39, 0, 7], dtype=torch.int32, device=DEV)
+    x = torch.empty(3, 32, device=DEV)
+    ops.embed(ids, where, wte, pos.embed_table(), x)
+    want = P.embed([3, 99, 0], [39, 0, 7], wte.double().cpu().numpy(), table.double().numpy())
+    assert np.abs(x.double().cpu().numpy() - want).max() < 1e-6
+    with pytest.raises(ValueError, match="rows"):
+        build_position(PositionSpec("learned", 41), {"table": table}, torch.bfloat16, DEV)
+    assert build_position(PositionSpec("none"), {}, torch.bfloat16, DEV).embed_table() is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("act,inner", [("gelu_new", 256), ("gelu", 200), ("relu", 72), ("silu", 136)])
+def test_feed_forward_part(dtype, act, inner):
+    from deliverance_amd.config import DenseFeedForwardSpec
+    from deliverance_amd.parts import build_feed_forward
+    g = torch.Generator().manual_seed(2)
+    E, N = 96, 7
+    p = {"fc_weight": (torch.randn(inner, E, generator=g) * 0.2).to(torch.bfloat16), "fc_bias": torch.randn(inner, generator=g).to(torch.bfloat16),
+         "proj_weight": (torch.randn(E, inner, generator=g) * 0.2).to(torch.bfloat16), "proj_bias": torch.randn(E, generator=g).to(torch.bfloat16)}
+    ff = build_feed_forward(DenseFeedForwardSpec("dense", E, inner, act), p, dtype, DEV)
+    ctx = make_ctx(dtype, [N], [0], 1, 16)
+    h = torch.randn(N, E, generator=g).to(dtype)
+    x0 = torch.randn(N, E, generator=g)
+    x = x0.clone().to(DEV)
+    ff.forward(ctx, h.to(DEV), x)
+    d = lambda t: t.double().numpy()
+    mid = P.ACTIVATIONS[act](d(h) @ d(p["fc_weight"]).T + d(p["fc_bias"]))
+    want = d(x0) + mid @ d(p["proj_weight"]).T + d(p["proj_bias"])
+    assert np.abs(x.double().cpu().numpy() - want).max() < TOL[dtype] * 3
+    with pytest.raises(ValueError, match="fc weight"):
+        build_feed_forward(DenseFeedForwardSpec("dense", E, inner + 8, act), p, dtype, DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,window", [(4, 4, 16, None), (6, 2, 48, None), (3, 3, 64, 20)])
+def test_attention_mixer_part(dtype, Hq, Hkv, D, window):
+    """Two steps: a whole prompt, then a mix of one decode token and a portion for another sequence."""
+    from deliverance_amd.config import AttentionSpec, LayerCall
+    from deliverance_amd.parts import build_mixer
+    g = torch.Generator().manual_seed(3)
+    E = 80
+    qkv_cols = (Hq + 2 * Hkv) * D
+    scale = 0.9 / math.sqrt(D)
+    p = {"qkv_weight": (torch.randn(qkv_cols, E, generator=g) * 0.3).to(torch.bfloat16), "qkv_bias": (torch.randn(qkv_cols, generator=g) * 0.3).to(torch.bfloat16),
+         "out_weight": (torch.randn(E, Hq * D, generator=g) * 0.2).to(torch.bfloat16), "out_bias": torch.randn(E, generator=g).to(torch.bfloat16)}
+    mixer = build_mixer(AttentionSpec("attention", E, Hq, Hkv, D, scale, window=window), p, dtype, DEV)
+    need = mixer.cache_need()
+    assert (need.n_kv_heads, need.head_dim, need.window) == (Hkv, D, window)
+    d = lambda t: t.double().numpy()
+    T = [37, 22]
+    hs = [torch.randn(t, E, generator=g).to(dtype) for t in T]
+
+    def plain(h):
+        qkv = d(h) @ d(p["qkv_weight"]).T + d(p["qkv_bias"])
+        if dtype == torch.bfloat16:
+            qkv = torch.tensor(qkv).to(torch.bfloat16).double().numpy()      # what the cache holds
+        q, k, v = qkv[:, :Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:]
+        o = P.causal_attention(q, k, v, Hq, scale, window=window, n_kv_head=Hkv)
+        return o @ d(p["out_weight"]).T + d(p["out_bias"])
+    want = [plain(h) for h in hs]
+    # step 1: sequence 0 brings 36 tokens, sequence 1 brings 15 -- both whole so far
+    ctx = make_ctx(dtype, [36, 15], [0, 0], Hkv, D, window=window)
+    h1 = torch.cat([hs[0][:36], hs[1][:15]]).to(DEV)
+    x = torch.zeros(51, E, device=DEV)
+    mixer.forward(ctx, h1, x, LayerCall(0, 0, True))
+    got = x.double().cpu().numpy()
+    assert np.abs(got[:36] - want[0][:36]).max() < TOL[dtype] * 4
+    assert np.abs(got[36:] - want[1][:15]).max() < TOL[dtype] * 4
+    # step 2 on the same cache: one decode token for sequence 0 beside a portion of 7 for sequence 1
+    ctx2 = make_ctx(dtype, [1, 7], [36, 15], Hkv, D, window=window)
+    ctx2.cache, ctx2.block_tables = ctx.cache, ctx2.block_tables
+    # reuse the pages of step 1 and extend them
+    bt_old, bt_new = ctx.block_tables[0].cpu(), ctx2.block_tables[0].cpu()
+    for s in range(2):
+        n_old = int((bt_old[s] >= 0).sum())
+        bt_new[s, :n_old] = bt_old[s, :n_old]
+    ctx2.block_tables = [bt_new.to(DEV)]
+    page = 16
+    slots = [int(bt_new[0, 36 // page]) * page + 36 % page] + [int(bt_new[1, (15 + i) // page]) * page + (15 + i) % page for i in range(7)]
+    ctx2.slot_maps = [torch.tensor(slots, dtype=torch.int32, device=DEV)]
+    ctx2.cache = SimpleNamespace(kv={0: torch.cat([ctx.cache.kv[0], torch.full_like(ctx.cache.kv[0], float("nan"))])},
+                                 group_of_slot={0: 0})
+    h2 = torch.cat([hs[0][36:37], hs[1][15:22]]).to(DEV)
+    x2 = torch.zeros(8, E, device=DEV)
+    mixer.forward(ctx2, h2, x2, LayerCall(0, 0, True))
+    got2 = x2.double().cpu().numpy()
+    assert np.abs(got2[0] - want[0][36]).max() < TOL[dtype] * 4
+    assert np.abs(got2[1:] - want[1][15:22]).max() < TOL[dtype] * 4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_part_and_fused_small_steps(model_b, dtype):
+    """A whole block from its spec, on a long step (separate kernels) and on a short one (the norm
+    fused into the products) -- both against the plain block."""
+    from deliverance_amd.config import Gpt2Config, LayerCall
+    from deliverance_amd.models import gpt2 as arch
+    from deliverance_amd.parts import Block
+    from deliverance_amd.weights import load_declared
+    import helpers
+    mc = Gpt2Config.from_dict(helpers.CONFIG_B).to_model_config()
+    bound = arch.bind_tensors(mc, load_declared(model_b.folder, arch.declare_tensors(mc)))
+    layer = 2
+    blk = Block(mc.layers[layer], bound["layers"][layer], dtype, DEV)
+    g = torch.Generator().manual_seed(4)
+    for T in (40, 5):
+        x0 = torch.randn(T, 96, generator=g)
+        ctx = make_ctx(dtype, [T], [0], 2, 48)
+        x = x0.clone().to(DEV)
+        blk.forward(ctx, x, LayerCall(layer, 0, True))
+        want = P.block(x0.double().numpy(), model_b.W, layer, model_b.plain_cfg)
+        assert np.abs(x.double().cpu().numpy() - want).max() < TOL[dtype] * 2, T
