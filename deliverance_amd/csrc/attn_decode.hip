@@ -60,7 +60,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   float m = -INFINITY, l = 0.f;
 
   for (int c0 = (lo / DA_WAVE) * DA_WAVE + wave * DA_WAVE; c0 <= p; c0 += DEC_WAVES * DA_WAVE) {
-    // ---- scores: iteration i handles keys c0 + i*G + sub; all loads first, then the arithmetic
+    // ---- all loads of the chunk first: the key pieces of the score phase and the value groups
+    // of the weighted sum (both need only the block table), then the arithmetic
     float mine = -INFINITY;      // one key's score per lane, once the loop is done
     uint4 kv[CPR];
     const int safe_key = p;      // a row that surely exists, read in place of rows that are not seen
@@ -71,6 +72,21 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       const int kk = valid ? key : safe_key;
       const bf16_t* kr = cache + cache_k_row(bt[kk / page], hk, kk % page, Hkv, page, D) + (piece_ok ? piece * 8 : 0);
       kv[i] = *(const uint4*)kr;
+    }
+    const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
+    const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
+    // the chunk's 8 groups of 8 keys (a group never crosses a page) of this lane's first dimension;
+    // groups with no seen key read the group of `last` instead and are dropped
+    uint4 vv0[8];
+    {
+      const int d = lane < D ? lane : 0;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const int g0 = c0 + g * 8;
+        const bool any = g0 + 7 >= first && g0 <= last;
+        const int gs = any ? g0 : (last / 8) * 8;
+        vv0[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+      }
     }
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
@@ -97,26 +113,27 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     l = l * alpha + wave_sum(e);
     m = m_new;
     ps[wave][kidx] = e;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the value loads stay in flight
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     // ---- values: lane owns dimensions lane, lane + 64, ...
-    const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
-    const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
 #pragma unroll
     for (int i = 0; i < DEC_DPL; ++i) {
       const int d = lane + i * DA_WAVE;
       if (d >= D) break;
       float a = acc[i] * alpha;
-      // the chunk's 8 groups of 8 keys (a group never crosses a page); groups with no seen key
-      // read the group of `last` instead and are dropped
       uint4 vv[8];
+      if (i == 0) {
 #pragma unroll
-      for (int g = 0; g < 8; ++g) {
-        const int g0 = c0 + g * 8;
-        const bool any = g0 + 7 >= first && g0 <= last;
-        const int gs = any ? g0 : (last / 8) * 8;
-        vv[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+        for (int g = 0; g < 8; ++g) vv[g] = vv0[g];
+      } else {
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+          const int g0 = c0 + g * 8;
+          const bool any = g0 + 7 >= first && g0 <= last;
+          const int gs = any ? g0 : (last / 8) * 8;
+          vv[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+        }
       }
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
@@ -136,9 +153,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       }
       acc[i] = a;
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the value loads stay in flight
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
 #pragma unroll
   for (int i = 0; i < DEC_DPL; ++i) {

@@ -86,6 +86,14 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// A workgroup barrier that orders LDS traffic only: loads from global memory that were issued
+// before it stay in flight across it (a full __syncthreads waits for them).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // The activations of a feed-forward, in 32-bit
 // (math/src/main/java/io/teknek/deliverance/math/ActivationFunction.java:13-21).
 __device__ __forceinline__ float apply_act(float x, int act) {

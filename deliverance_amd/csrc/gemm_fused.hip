@@ -61,6 +61,32 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
   const int n0 = blockIdx.x * FZ_COLS;
   const int fr = lane % 16, fk = (lane / 16) * 8;
 
+  // The first chunks of w and of the norm's gain and bias do not depend on the statistics: their
+  // loads are issued first and fly while the rows are read and reduced.
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const bool wrow_ok = n0 + fr < N;
+  const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
+  uint4 wv[FZ_UNROLL];
+  float gg[FZ_UNROLL][8], bb[FZ_UNROLL][8];
+  auto load_wgb = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < FZ_UNROLL; ++u) {
+      const int k = k0 + u * NW * 32;
+      const bool kin = k + fk < K;
+      const int ks = kin ? k : -fk;
+      wv[u] = load16(wp + ks);
+      if (!(kin && wrow_ok)) wv[u] = zero;
+      load8_param(ln.g, ln.g_dtype, ks + fk, gg[u]);
+      if (ln.b) load8_param(ln.b, ln.b_dtype, ks + fk, bb[u]);
+    }
+  };
+  load_wgb(wave * 32);
+  // what the epilogue needs, also early: this thread's output element is (em, ec)
+  const int em = t / FZ_COLS, ec = t % FZ_COLS;      // valid while t < MT * 16 * FZ_COLS
+  const bool e_ok = t < MT * 16 * FZ_COLS && em < M && n0 + ec < N;
+  const float e_bias = (e_ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n0 + ec) : 0.f;
+  const int e_slot = (e_ok && kv.cache) ? kv.slot_map[em] : -1;
+
   // ---- statistics of every row: wavefront v takes rows v, v + NW, ...
   for (int m = wave; m < M; m += NW) {
     const float* xr = ln.x + (size_t)(ln.rows ? ln.rows[m] : m) * K;
@@ -85,7 +111,7 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
     const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)K + ln.eps);
     if (lane == 0) { s_mean[m] = mean; s_rstd[m] = rstd; }
   }
-  __syncthreads();
+  lds_barrier();
 
   floatx4 acc[MT];
   float mean[MT], rstd[MT];
@@ -100,23 +126,14 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
     mean[i] = s_mean[ms]; rstd[i] = s_rstd[ms];
     xp[i] = ln.x + (size_t)(ln.rows ? ln.rows[ms] : ms) * K + fk;
   }
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  const bool wrow_ok = n0 + fr < N;
-  const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
 
   for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * FZ_UNROLL) {
-    uint4 wv[FZ_UNROLL];
+    if (k0 != wave * 32) load_wgb(k0);
     float4 xa[FZ_UNROLL][MT][2];
-    float gg[FZ_UNROLL][8], bb[FZ_UNROLL][8];
 #pragma unroll
     for (int u = 0; u < FZ_UNROLL; ++u) {
       const int k = k0 + u * NW * 32;
-      const bool kin = k + fk < K;
-      const int ks = kin ? k : -fk;
-      wv[u] = load16(wp + ks);
-      if (!(kin && wrow_ok)) wv[u] = zero;
-      load8_param(ln.g, ln.g_dtype, ks + fk, gg[u]);
-      if (ln.b) load8_param(ln.b, ln.b_dtype, ks + fk, bb[u]);
+      const int ks = (k + fk < K) ? k : -fk;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
         xa[u][i][0] = *(const float4*)(xp[i] + ks);
@@ -150,26 +167,21 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
-  __syncthreads();
-  for (int e = t; e < MT * 16 * FZ_COLS; e += NW * 64) {
-    const int m = e / FZ_COLS, c = e % FZ_COLS, n = n0 + c;
-    if (m < M && n < N) {
-      float v = red[0][m][c];
+  lds_barrier();
+  static_assert(MT * 16 * FZ_COLS <= NW * 64, "one output element per thread");
+  if (e_ok) {
+    const int n = n0 + ec;
+    float v = red[0][em][ec];
 #pragma unroll
-      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][m][c];
-      const float bias = ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
-      epilogue_store(ep, m, n, v, bias);
-      if (kv.cache && n >= kv.q_cols) {
-        const int slot = kv.slot_map[m];
-        if (slot >= 0) {
-          const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
-          const int h = cc / kv.D, d = cc % kv.D, pg = slot / kv.page, row = slot % kv.page;
-          const bf16_t val = f32_to_bf16(apply_act(v + bias, ep.act));
-          bf16_t* cache = (bf16_t*)kv.cache;
-          if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = val;
-          else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = val;
-        }
-      }
+    for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
+    epilogue_store(ep, em, n, v, e_bias);
+    if (kv.cache && n >= kv.q_cols && e_slot >= 0) {
+      const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
+      const int h = cc / kv.D, d = cc % kv.D, pg = e_slot / kv.page, row = e_slot % kv.page;
+      const bf16_t val = f32_to_bf16(apply_act(v + e_bias, ep.act));
+      bf16_t* cache = (bf16_t*)kv.cache;
+      if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = val;
+      else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = val;
     }
   }
 }
@@ -203,9 +215,8 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
   dim3 grid(da_ceil_div(N, FZ_COLS));
   const int mt = da_ceil_div(M, 16);
   hipStream_t s = (hipStream_t)stream;
-  if (K >= 2048) launch_fused<16>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
-  else if (K >= 1024) launch_fused<8>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
-  else launch_fused<4>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  if (K >= 1024) launch_fused<16>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  else launch_fused<8>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
   DA_CHECK_LAUNCH("gemm_bf16_ln");
   return 0;
 }

@@ -144,6 +144,16 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
     arow_ok[i] = i * 16 + fr < M;
     ap[i] = a + (size_t)(arow_ok[i] ? i * 16 + fr : 0) * lda + fk;
   }
+  // what the epilogue needs is asked for first, so that it has arrived when the products are done
+  constexpr int EPT = (MT * 16 * SK_COLS + NW * 64 - 1) / (NW * 64);     // output elements per thread
+  float e_bias[EPT], e_old[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = t + j * NW * 64, m = e / SK_COLS, n = n0 + e % SK_COLS;
+    const bool ok = e < MT * 16 * SK_COLS && m < M && n < N;
+    e_bias[j] = (ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
+    e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
+  }
   for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * SK_UNROLL) {
     uint4 wv[SK_UNROLL], av[SK_UNROLL][MT];
 #pragma unroll
@@ -170,14 +180,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
-  __syncthreads();
-  for (int e = t; e < MT * 16 * SK_COLS; e += NW * 64) {
-    const int m = e / SK_COLS, c = e % SK_COLS, n = n0 + c;
-    if (m < M && n < N) {
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = t + j * NW * 64, m = e / SK_COLS, c = e % SK_COLS, n = n0 + c;
+    if (e < MT * 16 * SK_COLS && m < M && n < N) {
       float v = red[0][m][c];
 #pragma unroll
       for (int v2 = 1; v2 < NW; ++v2) v += red[v2][m][c];
-      epilogue_store(ep, m, n, v, ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f);
+      v = apply_act(v + e_bias[j], ep.act);
+      const size_t o = (size_t)m * ep.ldo + n;
+      if (ep.accumulate) ((float*)ep.out)[o] = e_old[j] + v;
+      else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
+      else ((float*)ep.out)[o] = v;
     }
   }
 }
