@@ -81,25 +81,29 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 
   for (int kt = (b_lo / PF_BK) * PF_BK; kt <= b_last; kt += PF_BK) {
     // ---- stage the tile: keys kt .. kt+63, only those in b_lo .. b_last are read, the rest is zero
+    // Loads are unconditional (a conditional load becomes a branch that serialises them): a key
+    // outside b_lo .. b_last reads key b_last instead and is replaced by zero.
     for (int c = t; c < PF_BK * (D / 8); c += PF_WAVES * DA_WAVE) {
       const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (key >= b_lo && key <= b_last)
-        v = *(const uint4*)(cache + cache_k_row(bt[key / page], hk, key % page, Hkv, page, D) + pc * 8);
+      const bool ok = key >= b_lo && key <= b_last;
+      const int ks = ok ? key : b_last;
+      uint4 v = *(const uint4*)(cache + cache_k_row(bt[ks / page], hk, ks % page, Hkv, page, D) + pc * 8);
+      if (!ok) v = make_uint4(0, 0, 0, 0);
       *(uint4*)&Ks[kr * KLD + pc * 8] = v;
     }
     for (int c = t; c < DT * 32 * (PF_BK / 8); c += PF_WAVES * DA_WAVE) {
       const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;   // 8 keys of one dimension
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (d < D && key0 + 7 >= b_lo && key0 <= b_last) {
-        v = *(const uint4*)(cache + cache_v_base(bt[key0 / page], hk, Hkv, page, D) + (long long)d * page + key0 % page);
-        if (key0 < b_lo || key0 + 7 > b_last) {        // rows outside were never written for us
-          uint32_t u[4] = {v.x, v.y, v.z, v.w};
+      const bool ok = d < D && key0 + 7 >= b_lo && key0 <= b_last;
+      const int ks = ok ? key0 : (b_last / 8) * 8;
+      const int ds = d < D ? d : 0;
+      uint4 v = *(const uint4*)(cache + cache_v_base(bt[ks / page], hk, Hkv, page, D) + (long long)ds * page + ks % page);
+      if (!ok) v = make_uint4(0, 0, 0, 0);
+      if (key0 < b_lo || key0 + 7 > b_last) {          // rows outside were never written for us
+        uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (key0 + e < b_lo || key0 + e > b_last) u[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
-          v = make_uint4(u[0], u[1], u[2], u[3]);
-        }
+        for (int e = 0; e < 8; ++e)
+          if (key0 + e < b_lo || key0 + e > b_last) u[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
+        v = make_uint4(u[0], u[1], u[2], u[3]);
       }
       *(uint4*)&Vs[d * PF_VLD + g * 8] = v;
     }

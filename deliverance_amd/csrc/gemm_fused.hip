@@ -95,7 +95,8 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 #pragma unroll
     for (int i = 0; i < FZ_VPL; ++i) {
       const int c = (lane + i * 64) * 4;
-      v[i] = c < K ? *(const float4*)(xr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+      v[i] = *(const float4*)(xr + (c < K ? c : 0));          // never a conditional load
+      if (c >= K) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
       s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     }
     const float mean = wave_sum(s) / (float)K;

@@ -6,7 +6,8 @@
 // or 32-bit (plain store or += for the residual stream).  Two kernels:
 //
 //  * gemm_tile: 128x128 block tile, 4 wavefronts of 64x64 (2x2 MFMA 32x32x16), operands staged
-//    through LDS with a register prefetch of the next K-slab.  For steps with many rows (prefill).
+//    through two LDS buffers with the slab after next already in flight.  For steps with many rows
+//    (prefill).
 //  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its
 //    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
 //    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
@@ -21,17 +22,26 @@
 #include "gemm_common.h"
 #include <stdlib.h>
 
-#define BM 128
-#define BN 128
 #define BKT 64               // k per slab
 #define LDS_LD (BKT + 8)     // padded row length in elements (144 bytes): spreads rows over banks
 
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256)
+// Block tile BM x BN, WM x WN wavefronts of (BM/WM) x (BN/WN) each.  Two LDS buffers: while slab k is
+// multiplied out of one, the loads of slab k+1 are in flight and are then parked in the other; one
+// barrier per slab.
+// ---------------------------------------------------------------------------------------------
+// OUTMODE: 0 bf16 store, 1 f32 store, 2 f32 +=.  ACT and OUTMODE are compile-time so that the
+// epilogue is straight-line code.
+template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
+__global__ void __launch_bounds__(WM * WN * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                  Epilogue ep, int M, int N, int K, int tiles_m, int tiles_n) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * LDS_LD];
+  constexpr int THREADS = WM * WN * 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;       // MFMA tiles per wavefront
+  constexpr int CA = BM * 8 / THREADS, CW = BN * 8 / THREADS; // 16-byte chunks per thread and slab
+  static_assert(BM * 8 % THREADS == 0 && BN * 8 % THREADS == 0, "tile does not split over the threads");
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_LD];
 
   // Blocks that follow each other in launch order land on different XCDs (8 of them, each with
   // its own L2).  Give each XCD a contiguous run of tiles, m fastest, so that the blocks of one
@@ -47,73 +57,133 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
-  const int wm = (wave % 2) * 64, wn = (wave / 2) * 64;
+  const int wm = (wave % WM) * (BM / WM), wn = (wave / WM) * (BN / WN);
 
-  floatx16 acc[2][2];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // each thread moves 4 chunks of 16 bytes of each operand per slab
-  uint4 ra[4], rw[4];
+  // Loads are never conditional (a conditional load becomes a branch that serialises the slab's
+  // loads): rows past the edge read the last row, chunks past K read chunk 0, and the value is
+  // replaced by zero afterwards.
+  uint4 ra[CA], rw[CW];
   const uint4 zero = make_uint4(0, 0, 0, 0);
+  const bf16_t* pa[CA];
+  const bf16_t* pw[CW];
+  bool oka[CA], okw[CW];
+#pragma unroll
+  for (int i = 0; i < CA; ++i) {
+    const int c = t + THREADS * i, row = m0 + c / 8;
+    oka[i] = row < M;
+    pa[i] = a + (size_t)(oka[i] ? row : M - 1) * lda + (c % 8) * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < CW; ++i) {
+    const int c = t + THREADS * i, row = n0 + c / 8;
+    okw[i] = row < N;
+    pw[i] = w + (size_t)(okw[i] ? row : N - 1) * ldw + (c % 8) * 8;
+  }
+  const int kc_t = (t % 8) * 8;                     // this thread's chunk offset inside a slab (THREADS % 8 == 0)
   auto fetch = [&](int k0) {
+    const bool kin = k0 + kc_t < K;
+    const int ks = kin ? k0 : 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = t + 256 * i, row = c / 8, kc = (c % 8) * 8;
-      const bool kin = k0 + kc < K;
-      ra[i] = (kin && m0 + row < M) ? load16(a + (size_t)(m0 + row) * lda + k0 + kc) : zero;
-      rw[i] = (kin && n0 + row < N) ? load16(w + (size_t)(n0 + row) * ldw + k0 + kc) : zero;
+    for (int i = 0; i < CA; ++i) {
+      ra[i] = load16(pa[i] + ks);
+      if (!(kin && oka[i])) ra[i] = zero;
+    }
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      rw[i] = load16(pw[i] + ks);
+      if (!(kin && okw[i])) rw[i] = zero;
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = t + 256 * i, row = c / 8, kc = (c % 8) * 8;
-      *(uint4*)&As[row * LDS_LD + kc] = ra[i];
-      *(uint4*)&Ws[row * LDS_LD + kc] = rw[i];
+    for (int i = 0; i < CA; ++i) {
+      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;
+      *(uint4*)&As[buf][row * LDS_LD + kc] = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;
+      *(uint4*)&Ws[buf][row * LDS_LD + kc] = rw[i];
     }
   };
-
   const int fr = lane % 32, fk = (lane / 32) * 8;
+  const int nslab = (K + BKT - 1) / BKT;
   fetch(0);
-  for (int k0 = 0; k0 < K; k0 += BKT) {
-    stash();
-    __syncthreads();
-    if (k0 + BKT < K) fetch(k0 + BKT);
+  stash(0);
+  lds_barrier();
+  for (int sidx = 0; sidx < nslab; ++sidx) {
+    const int buf = sidx & 1;
+    if (sidx + 1 < nslab) fetch((sidx + 1) * BKT);      // in flight while this slab is multiplied
 #pragma unroll
     for (int kk = 0; kk < BKT; kk += 16) {
-      bf16x8_t af[2], bf[2];
+      bf16x8_t af[TM], bf[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        af[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&As[(wm + i * 32 + fr) * LDS_LD + kk + fk]);
+      for (int i = 0; i < TM; ++i)
+        af[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&As[buf][(wm + i * 32 + fr) * LDS_LD + kk + fk]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        bf[j] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ws[(wn + j * 32 + fr) * LDS_LD + kk + fk]);
+      for (int j = 0; j < TN; ++j)
+        bf[j] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ws[buf][(wn + j * 32 + fr) * LDS_LD + kk + fk]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
-    __syncthreads();
+    if (sidx + 1 < nslab) stash(buf ^ 1);               // the other buffer was last read before the previous barrier
+    lds_barrier();
   }
 
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn + j * 32 + fr;
     if (n >= N) continue;
     const float b = ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-        if (m < M) epilogue_store(ep, m, n, acc[i][j][r], b);
+        if (m < M) {
+          const float v = apply_act(acc[i][j][r] + b, ACT);
+          const size_t o = (size_t)m * ep.ldo + n;
+          if (OUTMODE == 2) ((float*)ep.out)[o] += v;
+          else if (OUTMODE == 1) ((float*)ep.out)[o] = v;
+          else ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
+        }
       }
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int ACT>
+static void launch_tile_act(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
+                            int M, int N, int K) {
+  const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
+  const dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
+  if (ep.accumulate)
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+  else if (ep.out_dtype == DA_F32)
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+}
+
+template <int BM, int BN, int WM, int WN>
+static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
+                        int M, int N, int K) {
+  switch (ep.act) {
+    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, M, N, K); break;
+    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, M, N, K); break;
+    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, M, N, K); break;
+    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, M, N, K); break;
+    default: launch_tile_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, M, N, K); break;
   }
 }
 
@@ -235,9 +305,13 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     else if (nw == 4) launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
     else launch_skinny<2>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
   } else {
-    const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
-    hipLaunchKernelGGL(gemm_tile_kernel, dim3(tiles_m * tiles_n), dim3(256), 0, s, A, lda, W, ldw, ep, M, N, K,
-                       tiles_m, tiles_n);
+    // Smaller tiles where 128x128 tiles would leave compute units idle.  Every configuration sums a
+    // row's products in the same order (64-wide slabs, 16 at a time), so the choice does not change
+    // a result.
+    const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
+    if (tiles128 < 128) launch_tile<64, 64, 2, 2>(s, A, lda, W, ldw, ep, M, N, K);
+    else if (tiles128 < 256) launch_tile<128, 64, 4, 2>(s, A, lda, W, ldw, ep, M, N, K);
+    else launch_tile<128, 128, 4, 2>(s, A, lda, W, ldw, ep, M, N, K);
   }
   DA_CHECK_LAUNCH("gemm_bf16");
   return 0;

@@ -96,7 +96,8 @@ layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
-    v[i] = c < E ? *(const float4*)(xr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    v[i] = *(const float4*)(xr + (c < E ? c : 0));          // never a conditional load
+    if (c >= E) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
   }
   const float mean = wave_sum(s) / (float)E;
