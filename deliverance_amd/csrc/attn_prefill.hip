@@ -3,7 +3,7 @@
 // sees the keys lo_i .. past+i of the cache (earlier steps' keys and the portion's own, which were
 // written just before).
 //
-// One workgroup per (portion, query head, 128 query rows); 4 wavefronts of 32 rows each.  Keys
+// One workgroup per (portion, query head, 32 * W query rows); W wavefronts of 32 rows each.  Keys
 // come in aligned tiles of 64 through LDS: the key rows as they lie in the pages, the values as
 // they lie in the pages too (dimension-major: a row of the LDS tile is one dimension, 64 keys).
 // Per tile and wavefront, with MFMA 32x32x16:
@@ -18,16 +18,16 @@
 // A row's sums run over key tiles in ascending order starting at the aligned tile of its lo: the
 // order depends on the row's position (and window) only.
 #include "common.h"
+#include <stdlib.h>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-#define PF_WAVES 4
-#define PF_BQ 128          // query rows per workgroup
 #define PF_BK 64           // keys per tile
 #define PF_VLD (PF_BK + 8) // padded length of a value row in LDS
+#define PF_BT_MAX 2048      // block-table entries a workgroup keeps in LDS (more are read from memory)
 
-template <int D16>         // head size / 16
+template <int D16, int PF_WAVES>   // head size / 16; wavefronts (32 query rows each) per workgroup
 __global__ void __launch_bounds__(PF_WAVES * DA_WAVE)
 attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                     const int* __restrict__ block_table, int max_blocks,
@@ -37,8 +37,13 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   constexpr int D = D16 * 16;
   constexpr int DT = (D + 31) / 32;       // 32-dimension tiles of the output
   constexpr int KLD = D + 8;              // padded length of a key row in LDS
+  constexpr int PF_BQ = PF_WAVES * 32;    // query rows per workgroup
+  constexpr int THREADS = PF_WAVES * DA_WAVE;
+  constexpr int K_PIECES = PF_BK * (D / 8), V_PIECES = DT * 32 * (PF_BK / 8);   // 16-byte pieces of a tile
+  constexpr int NK = (K_PIECES + THREADS - 1) / THREADS, NV = (V_PIECES + THREADS - 1) / THREADS;  // per thread
   __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BK * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DT * 32 * PF_VLD];
+  __shared__ int bts[PF_BT_MAX];
 
   const int s = seq0 + blockIdx.z, h = blockIdx.y;
   const int row0 = q_start[s], T = q_start[s + 1] - row0;
@@ -77,26 +82,46 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   for (int i = 0; i < DT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY, l = 0.f;                 // running maximum (base-2 domain) and sum of weights
+  const float scale2 = scale * 1.4426950408889634f;
 
-  for (int kt = (b_lo / PF_BK) * PF_BK; kt <= b_last; kt += PF_BK) {
-    // ---- stage the tile: keys kt .. kt+63, only those in b_lo .. b_last are read, the rest is zero
-    // Loads are unconditional (a conditional load becomes a branch that serialises them): a key
-    // outside b_lo .. b_last reads key b_last instead and is replaced by zero.
-    for (int c = t; c < PF_BK * (D / 8); c += PF_WAVES * DA_WAVE) {
+  // The next tile's keys and values are asked for (into registers) before the current tile is
+  // multiplied, so their latency hides behind the arithmetic.  Loads are unconditional (a conditional
+  // load becomes a branch that serialises them): a key outside b_lo .. b_last reads a key that
+  // exists and is replaced by zero.
+  // The block table's entries for this workgroup's keys are copied to LDS once: a table entry read
+  // from memory in front of every tile would make the tile's loads wait for it, and that wait also
+  // drains the loads still in flight for the tiles before.
+  const int pg_lo = b_lo >> (31 - __builtin_clz(page)), pg_hi = b_last >> (31 - __builtin_clz(page));
+  const bool bt_local = pg_hi - pg_lo + 1 <= PF_BT_MAX;
+  if (bt_local)
+    for (int i = t; i <= pg_hi - pg_lo; i += THREADS) bts[i] = bt[pg_lo + i];
+  __syncthreads();
+  auto page_of = [&](int key_page) -> long long { return bt_local ? bts[key_page - pg_lo] : bt[key_page]; };
+  // Two register sets: while a tile is multiplied, the loads of the next two are in flight.
+  uint4 rk0[NK], rv0[NV], rk1[NK], rv1[NV];
+  const int lg = 31 - __builtin_clz(page);              // page is a power of two (checked on the host)
+  const long long page_elems = 2LL * Hkv * page * D;
+  const bf16_t* kbase = cache + (long long)hk * page * D;
+  const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
+  auto fetch = [&](uint4* rk, uint4* rv, int kt) {
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int c0 = t + i * THREADS, c = c0 < K_PIECES ? c0 : 0;
       const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
       const bool ok = key >= b_lo && key <= b_last;
       const int ks = ok ? key : b_last;
-      uint4 v = *(const uint4*)(cache + cache_k_row(bt[ks / page], hk, ks % page, Hkv, page, D) + pc * 8);
-      if (!ok) v = make_uint4(0, 0, 0, 0);
-      *(uint4*)&Ks[kr * KLD + pc * 8] = v;
+      rk[i] = *(const uint4*)(kbase + page_of(ks >> lg) * page_elems + (ks & (page - 1)) * D + pc * 8);
+      if (!ok) rk[i] = make_uint4(0, 0, 0, 0);
     }
-    for (int c = t; c < DT * 32 * (PF_BK / 8); c += PF_WAVES * DA_WAVE) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
       const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;   // 8 keys of one dimension
       const bool ok = d < D && key0 + 7 >= b_lo && key0 <= b_last;
       const int ks = ok ? key0 : (b_last / 8) * 8;
       const int ds = d < D ? d : 0;
-      uint4 v = *(const uint4*)(cache + cache_v_base(bt[ks / page], hk, Hkv, page, D) + (long long)ds * page + ks % page);
+      uint4 v = *(const uint4*)(vbase + page_of(ks >> lg) * page_elems + ds * page + (ks & (page - 1)));
       if (!ok) v = make_uint4(0, 0, 0, 0);
       if (key0 < b_lo || key0 + 7 > b_last) {          // rows outside were never written for us
         uint32_t u[4] = {v.x, v.y, v.z, v.w};
@@ -105,9 +130,36 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           if (key0 + e < b_lo || key0 + e > b_last) u[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
         v = make_uint4(u[0], u[1], u[2], u[3]);
       }
-      *(uint4*)&Vs[d * PF_VLD + g * 8] = v;
+      rv[i] = v;
     }
-    __syncthreads();
+  };
+  auto stash = [&](const uint4* rk, const uint4* rv) {
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int c = t + i * THREADS, kr = c / (D / 8), pc = c % (D / 8);
+      if (c < K_PIECES) *(uint4*)&Ks[kr * KLD + pc * 8] = rk[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = t + i * THREADS, d = c / (PF_BK / 8), g = c % (PF_BK / 8);
+      if (c < V_PIECES) *(uint4*)&Vs[d * PF_VLD + g * 8] = rv[i];
+    }
+  };
+  const int kt0 = (b_lo / PF_BK) * PF_BK;
+  fetch(rk0, rv0, kt0);
+  if (kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
+  int parity = 0;
+  for (int kt = kt0; kt <= b_last; kt += PF_BK, parity ^= 1) {
+    // this tile's registers go to LDS; the set is then free for the tile after next
+    if (parity == 0) {
+      stash(rk0, rv0);
+      lds_barrier();
+      if (kt + 2 * PF_BK <= b_last) fetch(rk0, rv0, kt + 2 * PF_BK);
+    } else {
+      stash(rk1, rv1);
+      lds_barrier();
+      if (kt + 2 * PF_BK <= b_last) fetch(rk1, rv1, kt + 2 * PF_BK);
+    }
 
     if (wave_on && kt <= w_last && kt + PF_BK - 1 >= w_lo) {
       floatx16 sc[2];
@@ -121,22 +173,36 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           sc[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kd], sc[ks], 0, 0, 0);
         }
       }
-      // scale, mask, running maximum
+      // Scale, mask, running maximum and weights.  Scores are kept in the base-2 domain
+      // (s * scale * log2 e), so that a weight costs one subtraction and one hardware exp2.  A tile
+      // that every row of the wavefront sees whole needs no mask at all.
+      const bool whole = kt + PF_BK - 1 <= w_first && (window <= 0 || kt >= w_last - window + 1);
       float tmax = -INFINITY;
+      if (whole) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kt + ks * 32 + 8 * (r / 4) + 4 * hf + (r % 4);
-          const bool vis = q_ok && key <= pq && key >= q_lo;
-          const float v = vis ? sc[ks][r] * scale : -INFINITY;
-          sc[ks][r] = v;
-          tmax = fmaxf(tmax, v);
-        }
+          for (int r = 0; r < 16; ++r) {
+            sc[ks][r] *= scale2;
+            tmax = fmaxf(tmax, sc[ks][r]);
+          }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kt + ks * 32 + 8 * (r / 4) + 4 * hf + (r % 4);
+            const bool vis = q_ok && key <= pq && key >= q_lo;
+            const float v = vis ? sc[ks][r] * scale2 : -INFINITY;
+            sc[ks][r] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DA_WAVE));
       const float m_new = fmaxf(m, tmax);
       const bool any = m_new != -INFINITY;             // a row that has seen no key yet keeps zeros
-      const float alpha = any ? expf(m - m_new) : 1.f;
+      const float m_use = any ? m_new : 0.f;           // -inf - 0 stays -inf: weight 0, never NaN
+      const float alpha = __builtin_amdgcn_exp2f(m - m_use);
       float tsum = 0.f;
       bf16x8_t pf[2][2];
 #pragma unroll
@@ -146,12 +212,10 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           uint32_t u[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float p0 = any ? expf(sc[ks][kb * 8 + 2 * e] - m_new) : 0.f;
-            const float p1 = any ? expf(sc[ks][kb * 8 + 2 * e + 1] - m_new) : 0.f;
-            const bf16_t b0 = f32_to_bf16(p0), b1 = f32_to_bf16(p1);
-            // the sum uses the rounded weights, the same ones that multiply the values
-            tsum += bf16_to_f32(b0) + bf16_to_f32(b1);
-            u[e] = (uint32_t)b0 | ((uint32_t)b1 << 16);
+            const float p0 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e] - m_use);
+            const float p1 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e + 1] - m_use);
+            tsum += p0 + p1;
+            u[e] = pack2_bf16(p0, p1);
           }
           pf[ks][kb] = __builtin_bit_cast(bf16x8_t, make_uint4(u[0], u[1], u[2], u[3]));
         }
@@ -175,7 +239,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[ks][kb], acc_o[i], 0, 0, 0);
           }
     }
-    __syncthreads();
+    lds_barrier();
   }
 
   if (q_ok) {
@@ -187,8 +251,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       for (int r4 = 0; r4 < 4; ++r4) {
         const int d = i * 32 + 8 * r4 + 4 * hf;
         if (d < D) {
-          uint32_t lo2 = (uint32_t)f32_to_bf16(acc_o[i][r4 * 4] * inv) | ((uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 1] * inv) << 16);
-          uint32_t hi2 = (uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 2] * inv) | ((uint32_t)f32_to_bf16(acc_o[i][r4 * 4 + 3] * inv) << 16);
+          const uint32_t lo2 = pack2_bf16(acc_o[i][r4 * 4] * inv, acc_o[i][r4 * 4 + 1] * inv);
+          const uint32_t hi2 = pack2_bf16(acc_o[i][r4 * 4 + 2] * inv, acc_o[i][r4 * 4 + 3] * inv);
           *(uint2*)(orow + d) = make_uint2(lo2, hi2);
         }
       }
@@ -202,26 +266,29 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && page > 0 && max_query_len >= 0, "attn_prefill: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_prefill: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attn_prefill: head size %d is not a multiple of 16 up to 256", D);
-  DA_REQUIRE(page % 8 == 0 && PF_BK % page == 0, "attn_prefill: page size %d must be 8, 16, 32 or 64", page);
+  DA_REQUIRE(page >= 8 && (page & (page - 1)) == 0 && PF_BK % page == 0, "attn_prefill: page size %d must be 8, 16, 32 or 64", page);
   DA_REQUIRE(q_ld >= Hq * D && out_ld >= Hq * D && q_ld % 8 == 0 && out_ld % 4 == 0, "attn_prefill: row lengths");
   DA_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)cache % 16 == 0) && ((uintptr_t)out % 8 == 0),
              "attn_prefill: operands must be 16-byte aligned");
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_prefill: bad window or block table");
   DA_REQUIRE(n_seqs <= 65535 && Hq <= 65535, "attn_prefill: too many sequences or heads for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
-  dim3 grid(da_ceil_div(max_query_len, PF_BQ), Hq, n_seqs), block(PF_WAVES * DA_WAVE);
+  const int waves = 4;
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(N)                                                                                         \
-  case N:                                                                                                 \
-    hipLaunchKernelGGL(attn_prefill_kernel<N>, grid, block, 0, st, (const bf16_t*)q, q_ld,                \
-                       (const bf16_t*)cache, block_table, max_blocks, q_start, seq_lens, seq0, Hq, Hkv,   \
-                       page, scale, window, (bf16_t*)out, out_ld);                                        \
+#define LAUNCH2(N, W)                                                                                     \
+  hipLaunchKernelGGL((attn_prefill_kernel<N, W>), dim3(da_ceil_div(max_query_len, 32 * W), Hq, n_seqs),   \
+                     dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
+                     max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld)
+#define LAUNCH(N)        \
+  case N:                \
+    LAUNCH2(N, 4);       \
     break;
   switch (D / 16) {
     LAUNCH(1) LAUNCH(2) LAUNCH(3) LAUNCH(4) LAUNCH(5) LAUNCH(6) LAUNCH(7) LAUNCH(8)
     LAUNCH(9) LAUNCH(10) LAUNCH(11) LAUNCH(12) LAUNCH(13) LAUNCH(14) LAUNCH(15) LAUNCH(16)
   }
 #undef LAUNCH
+#undef LAUNCH2
   DA_CHECK_LAUNCH("attn_prefill");
   return 0;
 }

@@ -54,6 +54,15 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return (bf16_t)(u >> 16);
 }
 
+// Two floats to two bfloat16 in one word (first in the low half), round to nearest even, by the
+// hardware's packed conversion.
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) float float2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const float2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <typename T> struct DTypeOf;
 template <> struct DTypeOf<float> { static const int value = DA_F32; };
 template <> struct DTypeOf<bf16_t> { static const int value = DA_BF16; };

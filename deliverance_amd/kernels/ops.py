@@ -224,13 +224,15 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 FUSED_LN_MAX_ROWS = 32
 FUSED_LN_MAX_K = 2048
+FUSED_LN_MAX_N = 16384      # every 16 output columns recompute the rows' statistics: not for a vocabulary
 
 
 def can_fuse_ln(n_rows: int, x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether ``linear_ln`` takes this step: few rows, bfloat16 weights, a width the kernel holds."""
     K = w.shape[1]
     return (_MODE == "tuned" and w.dtype == torch.bfloat16 and 0 < n_rows <= FUSED_LN_MAX_ROWS
-            and K % 8 == 0 and K <= FUSED_LN_MAX_K and w.stride(0) % 8 == 0 and x.dtype == torch.float32)
+            and K % 8 == 0 and K <= FUSED_LN_MAX_K and w.shape[0] <= FUSED_LN_MAX_N
+            and w.stride(0) % 8 == 0 and x.dtype == torch.float32)
 
 
 def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_weight: torch.Tensor,
