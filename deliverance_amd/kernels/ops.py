@@ -30,16 +30,68 @@ def _dt(t: torch.Tensor) -> int:
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+    return None if t is None else t.data_ptr()
+
+
+_PINNED_STREAM = None
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if _PINNED_STREAM is not None:
+        return _PINNED_STREAM
+    return torch.cuda.current_stream().cuda_stream
+
+
+class pinned_stream:
+    """Inside this context every kernel goes to the stream that was current on entry, without asking
+    torch again for each launch (a model step launches about a hundred kernels)."""
+
+    def __enter__(self):
+        global _PINNED_STREAM
+        self._old = _PINNED_STREAM
+        _PINNED_STREAM = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _PINNED_STREAM
+        _PINNED_STREAM = self._old
+        return False
 
 
 def _check(rc: int):
     if rc != 0:
         raise KernelError(build.load().da_last_error().decode())
+
+
+_VP, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+_ARGTYPES = {
+    "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _VP],
+    "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
+    "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_bf16_ln": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP,
+                        _I, _I, _I, _I, _I, _VP],
+    "da_kv_write": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _VP],
+    "da_attn_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_decode": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_prefill": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_sample": [_VP, _I, _I, _I, _VP, _VP, _VP],
+    "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
+}
+_LIB = None
+
+
+def _lib():
+    """The kernel library with its argument types declared (conversion is then cheap and checked)."""
+    global _LIB
+    if _LIB is None:
+        lib = build.load()
+        for name, types in _ARGTYPES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = types
+            fn.restype = ctypes.c_int
+        _LIB = lib
+    return _LIB
 
 
 def _need(cond: bool, msg: str):
@@ -69,7 +121,7 @@ def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
     _need(wte.is_contiguous() and wte.shape[1] == E, "embed: token table width differs from out")
     if wpe is not None:
         _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: position table width differs from out")
-    _check(build.load().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
+    _check(_lib().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
                                  _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, _stream()))
     return out
 
@@ -88,8 +140,8 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
         _need(R <= x.shape[0], "layernorm: more output rows than input rows")
     else:
         _need(rows.dtype == torch.int32 and rows.numel() >= R, "layernorm: rows must be int32 with R entries")
-    _check(build.load().da_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), _ptr(bias),
-                                     _dt(bias) if bias is not None else 0, ctypes.c_float(eps), _ptr(out),
+    _check(_lib().da_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), _ptr(bias),
+                                     _dt(bias) if bias is not None else 0, eps, _ptr(out),
                                      _dt(out), R, E, _stream()))
     return out
 
@@ -108,7 +160,7 @@ def linear_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], o
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
-    _check(build.load().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
+    _check(_lib().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
                                     _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
                                     _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
     return out
@@ -127,7 +179,7 @@ def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.Tensor
     _need(two == 2 and Hkv == n_kv_heads and D == head_dim, "kv_write: cache slot shape differs from the heads")
     _need(cache_slot.dtype == qkv.dtype, "kv_write: cache and activations differ in dtype")
     _need(slot_map.dtype == torch.int32 and slot_map.numel() >= N, "kv_write: slot_map must be int32 [N]")
-    _check(build.load().da_kv_write(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot),
+    _check(_lib().da_kv_write(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot),
                                     _ptr(slot_map), N, Hkv, D, page, _stream()))
 
 
@@ -148,9 +200,9 @@ def attention_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.
           "attention: block_table must be contiguous int32 [S, max_blocks]")
     _need(seq_of_token.dtype == torch.int32 and positions.dtype == torch.int32, "attention: ids must be int32")
     _need(seq_of_token.numel() >= N and positions.numel() >= N, "attention: fewer ids than rows")
-    _check(build.load().da_attn_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table),
+    _check(_lib().da_attn_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table),
                                     block_table.shape[1], _ptr(seq_of_token), _ptr(positions), N, n_heads, Hkv,
-                                    D, page, ctypes.c_float(scale), int(window or 0), _ptr(out), out.stride(0),
+                                    D, page, scale, int(window or 0), _ptr(out), out.stride(0),
                                     _stream()))
     return out
 
@@ -168,7 +220,7 @@ def sample(logits: torch.Tensor, params: torch.Tensor, out_tokens: torch.Tensor)
     _need(params.is_contiguous() and params.numel() >= R * SAMPLE_ROW_FLOATS and params.element_size() == 4,
           "sample: params must hold R records of 8 four-byte fields")
     _need(out_tokens.dtype == torch.int32 and out_tokens.numel() >= R, "sample: out must be int32 [R]")
-    _check(build.load().da_sample(_ptr(logits), logits.stride(0), R, V, _ptr(params), _ptr(out_tokens), _stream()))
+    _check(_lib().da_sample(_ptr(logits), logits.stride(0), R, V, _ptr(params), _ptr(out_tokens), _stream()))
     return out_tokens
 
 
@@ -181,7 +233,7 @@ def top_logprobs(logits: torch.Tensor, params: torch.Tensor, n: int, out_idx: to
     _need(0 < n <= V, "top_logprobs: n must be in [1, V]")
     _need(out_idx.dtype == torch.int32 and out_idx.numel() >= R * n and out_idx.is_contiguous(), "top_logprobs: out_idx")
     _need(out_lp.dtype == torch.float32 and out_lp.numel() >= R * n and out_lp.is_contiguous(), "top_logprobs: out_lp")
-    _check(build.load().da_top_logprobs(_ptr(logits), logits.stride(0), R, V, _ptr(params), n, _ptr(out_idx),
+    _check(_lib().da_top_logprobs(_ptr(logits), logits.stride(0), R, V, _ptr(params), n, _ptr(out_idx),
                                         _ptr(out_lp), _stream()))
 
 
@@ -216,7 +268,7 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
-    _check(build.load().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
+    _check(_lib().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
                                      _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
                                      _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
     return out
@@ -265,9 +317,9 @@ def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_w
         _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
               "linear_ln: slot_map must be int32 [rows]")
         _need(q_cols + 2 * kv_cols == N, "linear_ln: q|k|v columns do not add up to N")
-    _check(build.load().da_gemm_bf16_ln(
+    _check(_lib().da_gemm_bf16_ln(
         _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), _ptr(norm_bias),
-        _dt(norm_bias) if norm_bias is not None else 0, ctypes.c_float(eps), _ptr(w), w.stride(0), _ptr(bias),
+        _dt(norm_bias) if norm_bias is not None else 0, eps, _ptr(w), w.stride(0), _ptr(bias),
         _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0), n_rows, N, K,
         _ptr(kv_cache), _ptr(slot_map), q_cols, kv_cols, Hkv, D, page, _stream()))
     return out
@@ -309,9 +361,9 @@ def attention_decode(q: torch.Tensor, cache_slot: torch.Tensor, block_table: tor
     _need(q.shape[0] >= n_seqs and out.shape[0] >= n_seqs and block_table.shape[0] >= n_seqs,
           "attention_decode: fewer rows than sequences")
     _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= n_seqs, "attention_decode: seq_lens must be int32 [S]")
-    _check(build.load().da_attn_decode(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+    _check(_lib().da_attn_decode(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
                                        block_table.shape[1], _ptr(seq_lens), n_seqs, n_heads, Hkv, D, page,
-                                       ctypes.c_float(scale), int(window or 0), _ptr(out), out.stride(0), _stream()))
+                                       scale, int(window or 0), _ptr(out), out.stride(0), _stream()))
     return out
 
 
@@ -326,9 +378,9 @@ def attention_prefill(q: torch.Tensor, cache_slot: torch.Tensor, block_table: to
     _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= seq0 + n_seqs, "attention_prefill: seq_lens must be int32 [S]")
     _need(block_table.shape[0] >= seq0 + n_seqs, "attention_prefill: block table has fewer rows than sequences")
     _need(q.shape[0] == out.shape[0], "attention_prefill: q and out differ in rows")
-    _check(build.load().da_attn_prefill(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+    _check(_lib().da_attn_prefill(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
                                         block_table.shape[1], _ptr(q_start), _ptr(seq_lens), seq0, n_seqs,
-                                        max_query_len, n_heads, Hkv, D, page, ctypes.c_float(scale),
+                                        max_query_len, n_heads, Hkv, D, page, scale,
                                         int(window or 0), _ptr(out), out.stride(0), _stream()))
     return out
 

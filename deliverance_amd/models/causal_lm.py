@@ -74,6 +74,10 @@ class CausalLM:
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor], n_want: int) -> torch.Tensor:
         """Logits [n_want, V] (32-bit) of rows ``want_rows`` (int32, device) of this step."""
+        with ops.pinned_stream():
+            return self._forward(ctx, want_rows, n_want)
+
+    def _forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor], n_want: int) -> torch.Tensor:
         N = ctx.n_tokens
         x = ctx.buf("residual", N, self.config.width, torch.float32)
         ops.embed(ctx.tokens, ctx.positions, self.token_table, self.embed_position.embed_table(), x)
