@@ -24,5 +24,22 @@ __device__ __forceinline__ void epilogue_store(const Epilogue& ep, int m, int n,
   else ((float*)ep.out)[o] = v;
 }
 
+// For a fused q|k|v projection: the k and v columns of a row also go to the row's place in the
+// paged cache (keys row-major, values dimension-major; see common.h).
+struct KvScatter {
+  void* cache;          // null: no scatter
+  const int* slot_map;  // per row: page * page_size + row in page, or -1
+  int q_cols, kv_cols;  // k occupies columns [q_cols, q_cols + kv_cols), v the next kv_cols
+  int Hkv, D, page;
+};
+
+__device__ __forceinline__ void kv_scatter_store(const KvScatter& kv, int slot, int n, float v) {
+  const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
+  const int h = cc / kv.D, d = cc % kv.D, pg = slot / kv.page, row = slot % kv.page;
+  bf16_t* cache = (bf16_t*)kv.cache;
+  if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = f32_to_bf16(v);
+  else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = f32_to_bf16(v);
+}
+
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }
 

@@ -16,7 +16,6 @@
 #include "gemm_common.h"
 
 #define FZ_COLS 16
-#define FZ_UNROLL 4
 #define FZ_VPL 8          // float4 per lane when a row is held in registers: K <= 2048
 
 struct LnPrologue {
@@ -27,13 +26,6 @@ struct LnPrologue {
   const void* b;
   int b_dtype;
   float eps;
-};
-
-struct KvScatter {
-  void* cache;          // null: no scatter
-  const int* slot_map;
-  int q_cols, kv_cols;  // k occupies columns [q_cols, q_cols+kv_cols), v the next kv_cols
-  int Hkv, D, page;
 };
 
 __device__ __forceinline__ void load8_param(const void* p, int dtype, int i, float* o) {
@@ -51,7 +43,7 @@ __device__ __forceinline__ void load8_param(const void* p, int dtype, int i, flo
   }
 }
 
-template <int MT, int NW>
+template <int MT, int NW, int FZ_UNROLL>
 __global__ void __launch_bounds__(NW * 64)
 gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
                       int M, int N, int K) {
@@ -81,11 +73,17 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
     }
   };
   load_wgb(wave * 32);
-  // what the epilogue needs, also early: this thread's output element is (em, ec)
-  const int em = t / FZ_COLS, ec = t % FZ_COLS;      // valid while t < MT * 16 * FZ_COLS
-  const bool e_ok = t < MT * 16 * FZ_COLS && em < M && n0 + ec < N;
-  const float e_bias = (e_ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n0 + ec) : 0.f;
-  const int e_slot = (e_ok && kv.cache) ? kv.slot_map[em] : -1;
+  // what the epilogue needs, also early: this thread's output elements are e = t, t + THREADS, ...
+  constexpr int EPT = (MT * 16 * FZ_COLS + NW * 64 - 1) / (NW * 64);
+  float e_bias[EPT];
+  int e_slot[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = t + j * NW * 64, em = e / FZ_COLS, ec = e % FZ_COLS;
+    const bool ok = e < MT * 16 * FZ_COLS && em < M && n0 + ec < N;
+    e_bias[j] = (ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n0 + ec) : 0.f;
+    e_slot[j] = (ok && kv.cache) ? kv.slot_map[em] : -1;
+  }
 
   // ---- statistics of every row: wavefront v takes rows v, v + NW, ...
   for (int m = wave; m < M; m += NW) {
@@ -169,29 +167,24 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
   lds_barrier();
-  static_assert(MT * 16 * FZ_COLS <= NW * 64, "one output element per thread");
-  if (e_ok) {
-    const int n = n0 + ec;
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = t + j * NW * 64, em = e / FZ_COLS, ec = e % FZ_COLS, n = n0 + ec;
+    if (!(e < MT * 16 * FZ_COLS && em < M && n < N)) continue;
     float v = red[0][em][ec];
 #pragma unroll
     for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
-    epilogue_store(ep, em, n, v, e_bias);
-    if (kv.cache && n >= kv.q_cols && e_slot >= 0) {
-      const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
-      const int h = cc / kv.D, d = cc % kv.D, pg = e_slot / kv.page, row = e_slot % kv.page;
-      const bf16_t val = f32_to_bf16(apply_act(v + e_bias, ep.act));
-      bf16_t* cache = (bf16_t*)kv.cache;
-      if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = val;
-      else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = val;
-    }
+    epilogue_store(ep, em, n, v, e_bias[j]);
+    if (kv.cache && n >= kv.q_cols && e_slot[j] >= 0)
+      kv_scatter_store(kv, e_slot[j], n, apply_act(v + e_bias[j], ep.act));
   }
 }
 
-template <int NW>
+template <int NW, int UN>
 static void launch_fused(int mt, dim3 grid, hipStream_t s, const LnPrologue& ln, const bf16_t* W, int ldw,
                          const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
-  if (mt == 1) hipLaunchKernelGGL((gemm_ln_skinny_kernel<1, NW>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
-  else hipLaunchKernelGGL((gemm_ln_skinny_kernel<2, NW>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
+  if (mt == 1) hipLaunchKernelGGL((gemm_ln_skinny_kernel<1, NW, UN>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_ln_skinny_kernel<2, NW, UN>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
 }
 
 extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, int g_dtype, const void* b,
@@ -216,8 +209,9 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
   dim3 grid(da_ceil_div(N, FZ_COLS));
   const int mt = da_ceil_div(M, 16);
   hipStream_t s = (hipStream_t)stream;
-  if (K >= 1024) launch_fused<16>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
-  else launch_fused<8>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  // 8 wavefronts, two chunks in flight each: 125 registers, so two workgroups share a compute unit
+  // (deeper unrolling needs 168 and halves that; 16 wavefronts spill)
+  launch_fused<8, 2>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
   DA_CHECK_LAUNCH("gemm_bf16_ln");
   return 0;
 }

@@ -35,7 +35,7 @@
 template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                 Epilogue ep, int M, int N, int K, int tiles_m, int tiles_n) {
+                 Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
   constexpr int THREADS = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;       // MFMA tiles per wavefront
   constexpr int CA = BM * 8 / THREADS, CW = BN * 8 / THREADS; // 16-byte chunks per thread and slab
@@ -157,6 +157,10 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
           if (OUTMODE == 2) ((float*)ep.out)[o] += v;
           else if (OUTMODE == 1) ((float*)ep.out)[o] = v;
           else ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
+          if (OUTMODE == 0 && kv.cache && n >= kv.q_cols) {
+            const int slot = kv.slot_map[m];
+            if (slot >= 0) kv_scatter_store(kv, slot, n, v);
+          }
         }
       }
   }
@@ -164,26 +168,26 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
 
 template <int BM, int BN, int WM, int WN, int ACT>
 static void launch_tile_act(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                            int M, int N, int K) {
+                            const KvScatter& kv, int M, int N, int K) {
   const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
   const dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if (ep.accumulate)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else if (ep.out_dtype == DA_F32)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
 }
 
 template <int BM, int BN, int WM, int WN>
 static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                        int M, int N, int K) {
+                        const KvScatter& kv, int M, int N, int K) {
   switch (ep.act) {
-    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, M, N, K); break;
-    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, M, N, K); break;
-    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, M, N, K); break;
-    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, M, N, K); break;
-    default: launch_tile_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, M, N, K); break;
+    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    default: launch_tile_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
   }
 }
 
@@ -196,7 +200,7 @@ static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
 template <int MT, int NW, int SK_UNROLL>   // row tiles of 16, wavefronts, k-chunks in flight per wavefront
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                   Epilogue ep, int M, int N, int K) {
+                   Epilogue ep, KvScatter kv, int M, int N, int K) {
   __shared__ float red[NW][MT * 16][SK_COLS + 1];
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int n0 = blockIdx.x * SK_COLS;
@@ -217,12 +221,14 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   // what the epilogue needs is asked for first, so that it has arrived when the products are done
   constexpr int EPT = (MT * 16 * SK_COLS + NW * 64 - 1) / (NW * 64);     // output elements per thread
   float e_bias[EPT], e_old[EPT];
+  int e_slot[EPT];
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = t + j * NW * 64, m = e / SK_COLS, n = n0 + e % SK_COLS;
     const bool ok = e < MT * 16 * SK_COLS && m < M && n < N;
     e_bias[j] = (ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
     e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
+    e_slot[j] = (ok && kv.cache) ? kv.slot_map[m] : -1;
   }
   for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * SK_UNROLL) {
     uint4 wv[SK_UNROLL], av[SK_UNROLL][MT];
@@ -263,22 +269,24 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
       if (ep.accumulate) ((float*)ep.out)[o] = e_old[j] + v;
       else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
       else ((float*)ep.out)[o] = v;
+      if (kv.cache && n >= kv.q_cols && e_slot[j] >= 0) kv_scatter_store(kv, e_slot[j], n, v);
     }
   }
 }
 
 template <int NW>
 static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
-                          const Epilogue& ep, int M, int N, int K) {
+                          const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
   // few rows leave registers for more chunks in flight
-  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
-  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
-  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, M, N, K);
+  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
 }
 
 extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
                             int act, int accumulate, void* out, int out_dtype, int ldo, int M, int N, int K,
+                            void* kv_cache, const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
                             void* stream) {
   DA_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   DA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0,
@@ -287,8 +295,13 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   DA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_bf16: leading sizes too small");
   DA_REQUIRE(!accumulate || out_dtype == DA_F32, "gemm_bf16: accumulation needs a 32-bit output");
   DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16: unknown activation %d", act);
+  if (kv_cache) {
+    DA_REQUIRE(out_dtype == DA_BF16 && !accumulate && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N &&
+               page > 0, "gemm_bf16: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);
+  }
   if (M == 0) return 0;
   Epilogue ep{bias, bias_dtype, act, accumulate, out, out_dtype, ldo};
+  KvScatter kv{kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page};
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
@@ -300,18 +313,18 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     if (force_nw < 0) { const char* e = getenv("DA_SKINNY_NW"); force_nw = e ? atoi(e) : 0; }
     int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
     if (force_nw > 0) nw = force_nw;
-    if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
-    else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
-    else if (nw == 4) launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
-    else launch_skinny<2>(mt, grid, s, A, lda, W, ldw, ep, M, N, K);
+    if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else if (nw == 4) launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else launch_skinny<2>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
   } else {
     // Smaller tiles where 128x128 tiles would leave compute units idle.  Every configuration sums a
     // row's products in the same order (64-wide slabs, 16 at a time), so the choice does not change
     // a result.
     const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
-    if (tiles128 < 128) launch_tile<64, 64, 2, 2>(s, A, lda, W, ldw, ep, M, N, K);
-    else if (tiles128 < 256) launch_tile<128, 64, 4, 2>(s, A, lda, W, ldw, ep, M, N, K);
-    else launch_tile<128, 128, 4, 2>(s, A, lda, W, ldw, ep, M, N, K);
+    if (tiles128 < 128) launch_tile<64, 64, 2, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+    else if (tiles128 < 256) launch_tile<128, 64, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+    else launch_tile<128, 128, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
   }
   DA_CHECK_LAUNCH("gemm_bf16");
   return 0;

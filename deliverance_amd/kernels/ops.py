@@ -68,7 +68,7 @@ _ARGTYPES = {
     "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _VP],
     "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
     "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
-    "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gemm_bf16_ln": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP,
                         _I, _I, _I, _I, _I, _VP],
     "da_kv_write": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _VP],
@@ -255,9 +255,24 @@ def kernel_mode() -> str:
     return _MODE
 
 
+def _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, name):
+    """The cache-scatter arguments of a fused q|k|v projection (zeros when there is none)."""
+    if kv_cache is None:
+        return None, None, 0, 0, 0, 0, 0
+    _need(kv_cache.dim() == 5 and kv_cache.is_contiguous() and kv_cache.dtype == torch.bfloat16 and
+          out.dtype == torch.bfloat16, f"{name}: cache slot must be contiguous bfloat16 [pages,2,Hkv,page,D]")
+    _, _, Hkv, page, D = kv_cache.shape
+    _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
+          f"{name}: slot_map must be int32 [rows]")
+    _need(q_cols + 2 * Hkv * D == N, f"{name}: q|k|v columns do not add up to N")
+    return kv_cache.data_ptr(), slot_map.data_ptr(), q_cols, Hkv * D, Hkv, D, page
+
+
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
-    """out (+)= act(a @ w.T + bias) on the matrix cores; a, w bfloat16, K a multiple of 8."""
+                act: Optional[str] = None, accumulate: bool = False, kv_cache: Optional[torch.Tensor] = None,
+                slot_map: Optional[torch.Tensor] = None, q_cols: int = 0) -> torch.Tensor:
+    """out (+)= act(a @ w.T + bias) on the matrix cores; a, w bfloat16, K a multiple of 8.  With
+    ``kv_cache`` the columns from ``q_cols`` on (k | v) also go to the cache rows ``slot_map``."""
     _dev(a, w, bias, out)
     _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
     M, K = a.shape
@@ -268,15 +283,20 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
+    _need(kv_cache is None or not accumulate, "linear: a cache scatter goes with a plain store")
+    kvp = _kv_args(kv_cache, slot_map, q_cols, M, N, out, "linear_mfma")
     _check(_lib().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
-                                     _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
-                                     _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
+                               _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
+                               _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp, _stream()))
     return out
 
 
-FUSED_LN_MAX_ROWS = 32
-FUSED_LN_MAX_K = 2048
-FUSED_LN_MAX_N = 16384      # every 16 output columns recompute the rows' statistics: not for a vocabulary
+# Measured on MI355X: the fused kernel wins up to 8 rows and a width of 1024; beyond, the separate
+# norm and product are faster (every 16 output columns recompute the rows' statistics).
+FUSED_LN_MAX_ROWS = 8
+FUSED_LN_MAX_K = 1024
+FUSED_LN_MAX_N = 16384      # ... and never for a vocabulary
+FUSED_LN_KERNEL_MAX_ROWS = 32
 
 
 def can_fuse_ln(n_rows: int, x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -301,27 +321,19 @@ def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_w
     _need(x.shape[1] == K and norm_weight.numel() == K and (norm_bias is None or norm_bias.numel() == K),
           "linear_ln: widths differ")
     _need(w.dtype == torch.bfloat16, "linear_ln: w must be bfloat16")
-    _need(0 < n_rows <= FUSED_LN_MAX_ROWS and out.shape[0] >= n_rows and out.shape[1] == N, "linear_ln: bad row count")
+    _need(0 < n_rows <= FUSED_LN_KERNEL_MAX_ROWS and out.shape[0] >= n_rows and out.shape[1] == N, "linear_ln: bad row count")
     if rows is None:
         _need(x.shape[0] >= n_rows, "linear_ln: fewer rows in x than asked")
     else:
         _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "linear_ln: rows must be int32")
     _need(bias is None or bias.numel() == N, "linear_ln: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear_ln: unknown activation {act!r}")
-    Hkv = D = page = kv_cols = 0
-    if kv_cache is not None:
-        _need(kv_cache.dim() == 5 and kv_cache.is_contiguous() and kv_cache.dtype == torch.bfloat16 and
-              out.dtype == torch.bfloat16, "linear_ln: cache slot must be contiguous bfloat16 [pages,2,Hkv,page,D]")
-        _, _, Hkv, page, D = kv_cache.shape
-        kv_cols = Hkv * D
-        _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
-              "linear_ln: slot_map must be int32 [rows]")
-        _need(q_cols + 2 * kv_cols == N, "linear_ln: q|k|v columns do not add up to N")
+    kvp = _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, "linear_ln")
     _check(_lib().da_gemm_bf16_ln(
         _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), _ptr(norm_bias),
         _dt(norm_bias) if norm_bias is not None else 0, eps, _ptr(w), w.stride(0), _ptr(bias),
         _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0), n_rows, N, K,
-        _ptr(kv_cache), _ptr(slot_map), q_cols, kv_cols, Hkv, D, page, _stream()))
+        *kvp, _stream()))
     return out
 
 
@@ -331,12 +343,19 @@ def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
+           act: Optional[str] = None, accumulate: bool = False, kv_cache: Optional[torch.Tensor] = None,
+           slot_map: Optional[torch.Tensor] = None, q_cols: int = 0) -> torch.Tensor:
     """out (+)= act(a @ w.T + bias); picks the kernel by dtype and mode.  Shapes the matrix-core
-    kernel does not take (K not a multiple of 8) go to the plain kernel, which takes any."""
+    kernel does not take (K not a multiple of 8) go to the plain kernel, which takes any.  With
+    ``kv_cache`` the k | v columns (from ``q_cols`` on) are also written to the cache rows
+    ``slot_map``: in the product's epilogue on the matrix cores, by the write kernel otherwise."""
     if _MODE == "tuned" and _mfma_ok(a, w):
-        return linear_mfma(a, w, bias, out, act, accumulate)
-    return linear_ref(a, w, bias, out, act, accumulate)
+        return linear_mfma(a, w, bias, out, act, accumulate, kv_cache, slot_map, q_cols)
+    linear_ref(a, w, bias, out, act, accumulate)
+    if kv_cache is not None:
+        _, _, Hkv, _, D = kv_cache.shape
+        kv_write(out, q_cols, q_cols + Hkv * D, kv_cache, slot_map, Hkv, D)
+    return out
 
 
 def _attn_common(q, cache_slot, block_table, n_heads, out, name):

@@ -64,14 +64,19 @@ class CausalSelfAttention(Mixer):
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
         N = h.shape[0]
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
-        ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
-        if self.position is not None:
-            self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
-        if call.write:
-            ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
-                         self.n_kv_heads, self.head_dim)
+        if self.position is None and call.write:
+            # the new keys and values go to the cache in the projection's epilogue
+            ops.linear(h, self.qkv_weight, self.qkv_bias, qkv, kv_cache=slot, slot_map=ctx.slot_maps[group],
+                       q_cols=self.q_cols)
+        else:
+            ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
+            if self.position is not None:
+                self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
+            if call.write:
+                ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
+                             self.n_kv_heads, self.head_dim)
         self._attend(ctx, qkv, x, slot, group)
 
     def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int) -> None:

@@ -383,6 +383,30 @@ def test_fused_norm_product(ops, M, N, K, pdtype):
         assert (out.double() - ref).abs().max() < tol
 
 
+@pytest.mark.parametrize("M", [5, 40, 300])
+def test_product_writes_keys_and_values(ops, M):
+    """The skinny (M <= 64) and tile kernels scatter the k | v columns in their epilogue."""
+    g = torch.Generator().manual_seed(M)
+    Hq, Hkv, D, page, K = 5, 3, 48, 16, 104
+    N = (Hq + 2 * Hkv) * D
+    n_pages = (M + page - 1) // page + 2
+    a = bf(torch.randn(M, K, generator=g)).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
+    bias = bf(torch.randn(N, generator=g)).to(DEV)
+    perm = torch.randperm(n_pages * page, generator=g)[:M].to(torch.int32)
+    perm[M // 2] = -1
+    slots = perm.to(DEV)
+    c1 = torch.zeros(n_pages, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
+    c2 = torch.zeros_like(c1)
+    out1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    out2 = torch.empty_like(out1)
+    ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D)
+    ops.linear_mfma(a, w, bias, out2)
+    ops.kv_write(out2, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)
+    assert torch.equal(out1, out2)
+    assert torch.equal(c1, c2) and c1.abs().sum() > 0
+
+
 def test_fused_norm_product_writes_keys_and_values(ops):
     g = torch.Generator().manual_seed(11)
     Hq, Hkv, D, page, M, K = 6, 2, 48, 16, 9, 96
