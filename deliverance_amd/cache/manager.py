@@ -142,6 +142,10 @@ class CacheManager:
     def length(self, rid) -> int:
         return self._req(rid).length
 
+    def pending(self, rid) -> int:
+        """Positions reserved beyond ``length`` and not yet committed."""
+        return self._req(rid).pending
+
     def state_slot(self, rid) -> int:
         return self._req(rid).state_slot
 
@@ -184,12 +188,16 @@ class CacheManager:
         r.pending += n_new
         return start
 
-    def commit(self, rid) -> List[Tuple[int, int]]:
-        """The reserved positions now belong to the request.  Pages that every later query
+    def commit(self, rid, n: Optional[int] = None) -> List[Tuple[int, int]]:
+        """The reserved positions (the first ``n`` of them, when given: a later step may have
+        reserved more already) now belong to the request.  Pages that every later query
         has left behind (window groups) go back; returns them as (group, page)."""
         r = self._req(rid)
-        r.length += r.pending
-        r.pending = 0
+        k = r.pending if n is None else n
+        if not (0 <= k <= r.pending):
+            raise CacheError(f"request {rid!r}: cannot commit {k} of {r.pending} reserved positions")
+        r.length += k
+        r.pending -= k
         released = []
         for g, pool in enumerate(self.pools):
             first = self._first_live_page(g, r.length)     # the next query sits at r.length

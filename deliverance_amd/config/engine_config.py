@@ -23,6 +23,7 @@ class EngineConfig:
     max_chunk: int = 512               # largest prompt portion (the reference's maxBatchSize)
     state_slots: Optional[int] = None  # slots for fixed-size per-request state; None: max_num_seqs
     use_graphs: bool = True            # replay decode-only steps from captured HIP graphs
+    run_ahead: bool = True             # launch the next decode step before the running one's tokens are read
     device: str = "cuda:0"
 
     def __post_init__(self):

@@ -44,6 +44,31 @@ extern "C" int da_embed(const int* tokens, const int* positions, const void* wte
 }
 
 // ------------------------------------------------------------------------------------------
+// tokens[n] = sampled[src[n]] where src[n] >= 0: a step that is launched before the step before
+// it has been read takes those tokens from that step's sampled tokens on the device.
+// ------------------------------------------------------------------------------------------
+__global__ void take_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ src,
+                                   const int* __restrict__ sampled, int N, int n_sampled, int vocab) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  const int s = src[n];
+  if (s < 0 || s >= n_sampled) return;
+  int t = sampled[s];
+  t = t < 0 ? 0 : (t >= vocab ? vocab - 1 : t);       // a row that sampled nothing must not index outside the table
+  tokens[n] = t;
+}
+
+extern "C" int da_take_tokens(int* tokens, const int* src, const int* sampled, int N, int n_sampled, int vocab,
+                              void* stream) {
+  DA_REQUIRE(N >= 0 && n_sampled > 0 && vocab > 0, "take_tokens: bad sizes N=%d sampled=%d", N, n_sampled);
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(take_tokens_kernel, dim3(da_ceil_div(N, 64)), dim3(64), 0, (hipStream_t)stream, tokens, src,
+                     sampled, N, n_sampled, vocab);
+  DA_CHECK_LAUNCH("take_tokens");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // LayerNorm over rows of 32-bit x; one wave per row; mean and centred variance in 32-bit.
 //   y = (x - mean) / sqrt(var + eps) * w + b        (var biased, eps inside the root)
 // Reference: core/src/main/java/io/teknek/deliverance/generator/LayerNorm.java:127-150

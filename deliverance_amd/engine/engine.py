@@ -28,7 +28,7 @@ from ..profiler import InferenceProfiler
 from ..sampling.params import GeneratorParameters
 from ..sampling.sampler import RECORD_WORDS, device_record
 from .device_cache import DeviceCache
-from .scheduler import Request, Scheduled, Scheduler
+from .scheduler import RUNNING, Request, Scheduled, Scheduler
 from .step import StepEntry, StepRunner
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -45,6 +45,17 @@ class Response:
     top_logprobs: List[list] = field(default_factory=list)
     error: Optional[str] = None
     preemptions: int = 0
+
+
+class _InFlight:
+    """A step that has been launched: its batch, and where its sampled tokens arrive."""
+
+    def __init__(self, batch: List[Scheduled], samplers: List[Scheduled]):
+        self.batch = batch
+        self.samplers = samplers
+        self.tokens_host: Optional[torch.Tensor] = None      # pinned; valid once ``ready`` has passed
+        self.ready: Optional[torch.cuda.Event] = None
+        self.lp = None                                       # (indices, values) of the top log-probabilities
 
 
 class CausalLanguageModel:
@@ -72,7 +83,10 @@ class CausalLanguageModel:
                                    engine_config.max_chunk, on_open=self.cache.reset_state)
         self._next_id = 0
         self._callbacks: Dict[Hashable, Callable] = {}
-        self._sampled_dev = torch.empty(max(engine_config.max_num_seqs, 64), dtype=torch.int32, device=model.device)
+        self._inflight: Optional[_InFlight] = None
+        self._n_launched = 0
+        n = 2 * max(engine_config.max_num_seqs, 64)
+        self._token_bufs = [torch.empty(n, dtype=torch.int32, pin_memory=True) for _ in range(3)]
 
     # ---- lower level: requests and steps -------------------------------------------------------
     def add_request(self, prompt: Sequence[int], params: Optional[GeneratorParameters] = None,
@@ -89,24 +103,72 @@ class CausalLanguageModel:
         return rid
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._inflight is not None
 
     def step(self) -> List[Request]:
-        """One scheduler decision, one model step, one sampling call.  Returns the requests
-        that finished in this step."""
+        """One scheduler decision and one model step with its sampling.  Returns the requests
+        whose end became known in this call.
+
+        A step whose tokens are all sampled on the device may be left running when the call
+        returns.  The next call then first launches the step after it (taking its tokens from the
+        device, ``Scheduler.schedule_ahead``) and only then reads the older step's tokens, so
+        the host's work for one step runs beside the device's work for the step before.  When
+        the next step cannot be decided ahead, the older step is read first, as without this."""
+        done: List[Request] = []
+        if self._inflight is not None:
+            ahead = self._launch_ahead(self._inflight)
+            done += self._retire(self._inflight)
+            self._inflight = ahead
+            if ahead is not None:
+                return done
         before = len(self.scheduler.finished)
         with InferenceProfiler.timer("scheduler.schedule"):
             batch: List[Scheduled] = self.scheduler.schedule()
-        failed = self.scheduler.finished[before:]
+        done += self.scheduler.finished[before:]         # requests that failed in scheduling
         if not batch:
-            return list(failed)
+            return done
+        flight = self._launch(batch, None)
+        if self._may_stay_in_flight(flight):
+            self._inflight = flight
+        else:
+            done += self._retire(flight)
+        return done
+
+    def drain(self) -> List[Request]:
+        """Read the step that is still running, if there is one."""
+        if self._inflight is None:
+            return []
+        flight, self._inflight = self._inflight, None
+        return self._retire(flight)
+
+    def _may_stay_in_flight(self, flight: "_InFlight") -> bool:
+        return (self.engine_config.run_ahead and bool(flight.samplers) and flight.lp is None
+                and len(flight.samplers) == len(flight.batch))
+
+    def _launch_ahead(self, prev: "_InFlight") -> Optional["_InFlight"]:
+        if any(s.request.params.log_probs and s.request.params.top_log_probs > 0 for s in prev.batch):
+            return None
+        with InferenceProfiler.timer("scheduler.schedule"):
+            batch = self.scheduler.schedule_ahead(prev.batch)
+        if batch is None:
+            return None
+        row = {id(s.request): i for i, s in enumerate(prev.samplers)}
+        return self._launch(batch, row)
+
+    def _launch(self, batch: List[Scheduled], sampled_row: Optional[Dict[int, int]]) -> "_InFlight":
+        """Put one step on the device: model, sampling, and the copy of the sampled tokens to the
+        host.  With ``sampled_row`` every entry's token is the one the step before sampled for the
+        same request (row ``sampled_row[id(request)]`` of the runner's sampled tokens)."""
         V = self.config.vocab_size
         entries = []
         records: List[int] = []
         samplers: List[Scheduled] = []
         for s in batch:
             req = s.request
-            entries.append(StepEntry(req.rid, req.tokens_from(s.start, s.n), [s.n - 1] if s.samples else []))
+            if sampled_row is None:
+                entries.append(StepEntry(req.rid, req.tokens_from(s.start, s.n), [s.n - 1] if s.samples else []))
+            else:
+                entries.append(StepEntry(req.rid, [0], [0], from_sampled=sampled_row[id(req)]))
             if s.samples:
                 records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))
                 samplers.append(s)
@@ -114,40 +176,59 @@ class CausalLanguageModel:
         with InferenceProfiler.timer("generation.decode" if decode_only else "generation.prefill"):
             logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
         InferenceProfiler.counter("engine.batch_tokens", sum(s.n for s in batch))
+        flight = _InFlight(batch, samplers)
+        if not samplers:
+            return flight
+        R = len(samplers)
+        out = getattr(ctx, "sampled", None)           # a replayed graph has sampled already
+        if out is None:
+            out = self.runner.sampled[:R]
+            ops.sample(logits, ctx.extra, out)
+        want_lp = [s for s in samplers if s.request.params.log_probs and s.request.params.top_log_probs > 0]
+        if want_lp:
+            n = max(s.request.params.top_log_probs for s in want_lp)
+            idx = torch.empty((R, n), dtype=torch.int32, device=self.model.device)
+            val = torch.empty((R, n), dtype=torch.float32, device=self.model.device)
+            ops.top_logprobs(logits, ctx.extra, n, idx, val)
+            flight.lp = (idx, val)
+        host = self._token_bufs[self._n_launched % len(self._token_bufs)]
+        self._n_launched += 1
+        if host.numel() < R:
+            host = torch.empty(2 * R, dtype=torch.int32, pin_memory=True)
+            self._token_bufs[(self._n_launched - 1) % len(self._token_bufs)] = host
+        host[:R].copy_(out, non_blocking=True)
+        flight.tokens_host = host
+        flight.ready = torch.cuda.Event()
+        flight.ready.record()
+        return flight
+
+    def _retire(self, flight: "_InFlight") -> List[Request]:
+        """Wait for a launched step's tokens, book it with the scheduler, tell the callbacks."""
         sampled: Dict[Hashable, int] = {}
+        samplers = flight.samplers
         if samplers:
-            R = len(samplers)
-            if self._sampled_dev.numel() < R:
-                self._sampled_dev = torch.empty(2 * R, dtype=torch.int32, device=self.model.device)
-            out = getattr(ctx, "sampled", None)       # a replayed graph has sampled already
-            if out is None:
-                out = self._sampled_dev[:R]
-                ops.sample(logits, ctx.extra, out)
-            want_lp = [s for s in samplers if s.request.params.log_probs and s.request.params.top_log_probs > 0]
-            lp = None
-            if want_lp:
-                n = max(s.request.params.top_log_probs for s in want_lp)
-                idx = torch.empty((R, n), dtype=torch.int32, device=self.model.device)
-                val = torch.empty((R, n), dtype=torch.float32, device=self.model.device)
-                ops.top_logprobs(logits, ctx.extra, n, idx, val)
-                lp = (idx.cpu(), val.cpu())
             with InferenceProfiler.timer("sampler.sample"):
-                host = out.cpu()                               # the step's one synchronisation
+                flight.ready.synchronize()                   # the step's one synchronisation
+                host = flight.tokens_host[:len(samplers)].tolist()
+            lp = None if flight.lp is None else (flight.lp[0].cpu(), flight.lp[1].cpu())
             for i, s in enumerate(samplers):
-                sampled[s.request.rid] = int(host[i])
+                if s.request.state != RUNNING:
+                    continue                                 # ended while this step was running
+                sampled[s.request.rid] = host[i]
                 p = s.request.params
                 if lp is not None and p.log_probs and p.top_log_probs > 0:
                     k = p.top_log_probs
                     s.request.top_logprobs.append(list(zip(lp[0][i, :k].tolist(), lp[1][i, :k].tolist())))
-        done = self.scheduler.complete(batch, sampled)
+        live = [s for s in samplers if s.request.state == RUNNING]
+        done = self.scheduler.complete(flight.batch, sampled)
         now = time.perf_counter()
-        for s in samplers:
+        for s in live:
             cb = self._callbacks.get(s.request.rid)
             if cb is not None:
                 cb(sampled[s.request.rid], s.request.rid, (now - s.request.t_arrival) * 1e3)
         for r in done:
             self._callbacks.pop(r.rid, None)
-        return list(failed) + done
+        return done
 
     # ---- the entry point ---------------------------------------------------------------------
     def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],
@@ -176,6 +257,7 @@ class CausalLanguageModel:
             for r in self.step():
                 if r.rid in mine:
                     got[r.rid] = r
+        self.drain()                 # a step launched ahead for requests that have ended since
         out = [self._response(got[r]) for r in rids]
         for r in rids:
             self.scheduler.finished.remove(got[r])

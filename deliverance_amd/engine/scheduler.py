@@ -17,6 +17,10 @@ this engine's own:
   preempted: its pages go back and it returns to the head of the waiting queue to be computed
   again from its tokens (prompt and what it has generated).  A request that is alone and still
   cannot fit fails with ``finish_reason = "error"``.
+* ``schedule_ahead`` decides the step after one that is still running, before its tokens are
+  known, when that decision cannot depend on them: every running request gets its next decode
+  step, except those that end by length.  A request that turns out to have sampled an end token
+  has then one step too many in flight; its result is dropped when that step is booked.
 """
 from __future__ import annotations
 
@@ -203,6 +207,41 @@ class Scheduler:
             self.counters["batch_tokens"] += sum(s.n for s in batch)
         return batch
 
+    # ---- the step after a running one ----------------------------------------------------------
+    def _ends_by_length(self, req: Request, more: int) -> bool:
+        """Whether the request is done by its length once ``more`` further tokens are appended."""
+        p = req.params
+        return ((p.max_tokens is not None and len(req.output) + more >= p.max_tokens)
+                or req.n_tokens + more > req.limit)
+
+    def schedule_ahead(self, inflight: List[Scheduled]) -> Optional[List[Scheduled]]:
+        """The batch that follows ``inflight`` (scheduled, launched, not yet completed), or None
+        when it can only be decided after ``complete``: someone waits and could be admitted, a
+        running request is not at its last token in ``inflight``, or pages are short (preemption
+        needs the tokens).  Nothing is reserved when None is returned."""
+        if self.waiting and len(self.running) < self.max_num_seqs and self.cache.can_open():
+            return None
+        last = {id(s.request): s for s in inflight}
+        nxt: List[Request] = []
+        for req in self.running:
+            s = last.get(id(req))
+            if s is None or not s.samples or s.start + s.n != req.n_tokens:
+                return None
+            if not self._ends_by_length(req, 1):
+                nxt.append(req)
+        if not nxt or len(nxt) > self.max_batch_tokens:
+            return None
+        need = [0] * len(self.cache.pools)
+        for req in nxt:
+            for g, n in enumerate(self.cache.pages_needed(req.rid, 1)):
+                need[g] += n
+        if any(n > pool.n_free for n, pool in zip(need, self.cache.pools)):
+            return None
+        batch = [Scheduled(req, self.cache.extend(req.rid, 1), 1, True) for req in nxt]
+        self.counters["steps"] += 1
+        self.counters["batch_tokens"] += len(batch)
+        return batch
+
     # ---- after the step ----------------------------------------------------------------------
     def finish_check(self, req: Request, token: int) -> Optional[str]:
         """Stop rules after a token was appended (GenerationEngine.java:189-219,163-173):
@@ -228,7 +267,7 @@ class Scheduler:
             req = s.request
             if req.state != RUNNING:
                 continue
-            self.cache.commit(req.rid)
+            self.cache.commit(req.rid, s.n)           # a step scheduled ahead may hold a reservation of its own
             req.n_computed = s.start + s.n
             if not s.samples:
                 continue

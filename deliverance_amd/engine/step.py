@@ -26,6 +26,9 @@ class StepEntry:
     rid: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)    # places among ``tokens`` whose logits are wanted
+    # The entry's one token is not known on the host yet: it is row ``from_sampled`` of the tokens
+    # that the step before sampled on the device (``StepRunner.sampled``); ``tokens`` holds a placeholder.
+    from_sampled: Optional[int] = None
 
 
 class StepError(ValueError):
@@ -46,6 +49,9 @@ class StepRunner:
         self.use_graphs = use_graphs and model.graph_safe
         self.max_graph_batch = max_graph_batch
         self._graphs = {}
+        # where every sampling step leaves its tokens (row i: the i-th wanted row), and where a step
+        # launched on top of it takes them from
+        self.sampled = torch.zeros(2 * max(64, max_graph_batch), dtype=torch.int32, device=self.device)
 
     # ---- host -> device in one copy --------------------------------------------------------
     def _upload(self, words: List[int]) -> torch.Tensor:
@@ -72,7 +78,7 @@ class StepRunner:
         ``sample_records`` (8 words per wanted row, see sampling.device_record) ride along in the
         same host-to-device copy (``ctx.extra``); when they are given and the step holds one-token
         sequences only, the step and its sampling are replayed from a recorded HIP graph and the
-        sampled tokens are left in ``ctx.sampled``."""
+        sampled tokens are left in ``ctx.sampled`` (the first rows of ``self.sampled``)."""
         mgr = self.cache.manager
         cfg = self.model.config
         if not entries:
@@ -90,11 +96,15 @@ class StepRunner:
             for w in e.want:
                 if not (0 <= int(w) < len(e.tokens)):
                     raise StepError(f"request {e.rid!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+            if e.from_sampled is not None and not (len(e.tokens) == 1 and 0 <= e.from_sampled < self.sampled.numel()):
+                raise StepError(f"request {e.rid!r}: only a single token can come from the sampled tokens")
 
         starts = {}
         if reserved:
-            for e in entries:
-                starts[e.rid] = mgr.length(e.rid)
+            for e in entries:               # the entry's tokens are the last positions that were reserved
+                starts[e.rid] = mgr.length(e.rid) + mgr.pending(e.rid) - len(e.tokens)
+                if starts[e.rid] < mgr.length(e.rid):
+                    raise StepError(f"request {e.rid!r} brings {len(e.tokens)} tokens, {mgr.pending(e.rid)} are reserved")
         else:
             done = []
             opened = []
@@ -133,6 +143,9 @@ class StepRunner:
         ctx = self._context(dev, offs, meta, self.arena)
         self.last_ctx = ctx
         R = meta["R"]
+        if any(e.from_sampled is not None for e in entries):
+            from ..kernels import ops
+            ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, cfg.vocab_size)
         logits = self.model.forward(ctx, ctx.want_rows if R else None, R)
         if not reserved:                 # who reserves commits: the scheduler does it for its batches
             for e in entries:
@@ -148,6 +161,7 @@ class StepRunner:
         mgr = self.cache.manager
         S_real = len(entries)
         tokens: List[int] = []
+        token_src: List[int] = []
         positions: List[int] = []
         seq_of: List[int] = []
         q_start = [0]
@@ -159,6 +173,7 @@ class StepRunner:
             st = starts[e.rid]
             row0[i] = len(tokens)
             tokens += [int(t) for t in e.tokens]
+            token_src += [e.from_sampled] if e.from_sampled is not None else [-1] * len(e.tokens)
             positions += list(range(st, st + len(e.tokens)))
             seq_of += [s] * len(e.tokens)
             q_start.append(len(tokens))
@@ -167,18 +182,18 @@ class StepRunner:
         want_rows = [row0[i] + int(w) for i, e in enumerate(entries) for w in e.want]
         n_pad = 0 if pad_to is None else pad_to - S_real
         for k in range(n_pad):
-            tokens.append(0); positions.append(0); seq_of.append(S_real + k)
+            tokens.append(0); token_src.append(-1); positions.append(0); seq_of.append(S_real + k)
             q_start.append(len(tokens)); seq_lens.append(0); state_slots.append(-1)
             want_rows.append(len(tokens) - 1)
         N, S, R = len(tokens), S_real + n_pad, len(want_rows)
         G = len(self.cache.groups)
         if max_blocks is None:
             max_blocks = max(1, max(len(mgr.table(entries[i].rid, g)) for i in order for g in range(G))) if G else 1
-        words = tokens + positions + seq_of + q_start + seq_lens + state_slots + want_rows
+        words = tokens + token_src + positions + seq_of + q_start + seq_lens + state_slots + want_rows
         offs = {}
         o = 0
-        for name, n in (("tokens", N), ("positions", N), ("seq_of", N), ("q_start", S + 1), ("seq_lens", S),
-                        ("state_slots", S), ("want", R)):
+        for name, n in (("tokens", N), ("token_src", N), ("positions", N), ("seq_of", N), ("q_start", S + 1),
+                        ("seq_lens", S), ("state_slots", S), ("want", R)):
             offs[name] = (o, n)
             o += n
         for g in range(G):
@@ -213,6 +228,7 @@ class StepRunner:
         ctx.dtype = self.model.dtype
         ctx.n_tokens, ctx.n_seqs, ctx.n_decode = N, S, meta["n_decode"]
         ctx.tokens, ctx.positions, ctx.seq_of_token = view("tokens"), view("positions"), view("seq_of")
+        ctx.token_src = view("token_src")
         ctx.q_start, ctx.seq_lens, ctx.state_slots = view("q_start"), view("seq_lens"), view("state_slots")
         ctx.q_start_host, ctx.seq_lens_host, ctx.state_slots_host = meta["q_start"], meta["seq_lens"], meta["state_slots"]
         ctx.max_query_len = max(meta["q_start"][s + 1] - meta["q_start"][s] for s in range(S))
@@ -242,8 +258,7 @@ class StepRunner:
         if st is None:
             st = {"dev": torch.empty(len(words), dtype=torch.int32, device=self.device),
                   "host": torch.empty(len(words), dtype=torch.int32, pin_memory=True),
-                  "arena": Arena(self.device), "graph": None, "copied": None,
-                  "tokens": torch.empty(bucket, dtype=torch.int32, device=self.device)}
+                  "arena": Arena(self.device), "graph": None, "copied": None}
             self._graphs[bucket] = st
         assert st["dev"].numel() == len(words), "a bucket's layout is fixed"
         if st["copied"] is not None:
@@ -255,9 +270,12 @@ class StepRunner:
         ctx = self._context(st["dev"], offs, meta, st["arena"])
         self.last_ctx = ctx
 
+        sampled = self.sampled[:bucket]
+
         def body():
+            ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, self.model.config.vocab_size)
             logits = self.model.forward(ctx, ctx.want_rows, bucket)
-            ops.sample(logits, ctx.extra, st["tokens"])
+            ops.sample(logits, ctx.extra, sampled)
             return logits
 
         if st["graph"] is None:
@@ -270,5 +288,5 @@ class StepRunner:
             # the eager run above already did this step's work; the recorded graph is used from the next step on
         else:
             st["graph"].replay()
-        ctx.sampled = st["tokens"][:S]
+        ctx.sampled = sampled[:S]
         return st["logits"][:S], ctx

@@ -66,6 +66,7 @@ def _check(rc: int):
 _VP, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 _ARGTYPES = {
     "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _VP],
+    "da_take_tokens": [_VP, _VP, _VP, _I, _I, _I, _VP],
     "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
     "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
@@ -124,6 +125,16 @@ def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
     _check(_lib().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
                                  _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, _stream()))
     return out
+
+
+def take_tokens(tokens: torch.Tensor, src: torch.Tensor, sampled: torch.Tensor, vocab: int) -> torch.Tensor:
+    """tokens[n] = sampled[src[n]] wherever src[n] >= 0 (in place)."""
+    _dev(tokens, src, sampled)
+    _need(tokens.dtype == src.dtype == sampled.dtype == torch.int32, "take_tokens: int32 tensors needed")
+    _need(src.numel() >= tokens.numel(), "take_tokens: fewer sources than tokens")
+    _check(_lib().da_take_tokens(_ptr(tokens), _ptr(src), _ptr(sampled), tokens.numel(), sampled.numel(), int(vocab),
+                                 _stream()))
+    return tokens
 
 
 # ------------------------------------------------------------------------------- norms

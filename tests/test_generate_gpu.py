@@ -64,6 +64,40 @@ def test_replayed_graph_decodes_what_the_step_by_step_path_decodes(model_b):
     assert outs[True] == outs[False]
 
 
+@pytest.mark.parametrize("dtype,graphs", [("bfloat16", True), ("float32", False)])
+def test_steps_launched_ahead_decode_what_steps_read_one_by_one_decode(model_b, dtype, graphs):
+    """With run_ahead the next decode step is launched before the running one's tokens are read
+    (they are taken on the device); requests that end by length leave the batch in time, a request
+    that samples an end token has one step too many, whose result is dropped."""
+    from deliverance_amd import GeneratorParameters
+    m = model_b
+    prompts = [m.prompt(n, salt=7) for n in (4, 30, 11, 2, 50, 23)]
+    eng0 = load(m, dtype, use_graphs=graphs, run_ahead=False)
+    free = eng0.generate(prompts[3], GeneratorParameters(max_tokens=40, ignore_eos=True)).generated_tokens
+    eos = {free[10]}
+    params = [GeneratorParameters(max_tokens=20, ignore_eos=True), GeneratorParameters(max_tokens=5, ignore_eos=True),
+              GeneratorParameters(temperature=0.9, seed=77, top_k=40, max_tokens=33, ignore_eos=True),
+              GeneratorParameters(max_tokens=40), GeneratorParameters(ntokens=59, ignore_eos=True),
+              GeneratorParameters(temperature=0.7, seed=3, top_p=0.9, max_tokens=17, ignore_eos=True)]
+    outs = {}
+    for ahead in (False, True):
+        eng = load(m, dtype, use_graphs=graphs, run_ahead=ahead)
+        eng.scheduler.eos = eos
+        seen = []
+        res = eng.generate(prompts, params, on_token=lambda tok, i, ms: seen.append((i, tok)))
+        outs[ahead] = [(o.generated_tokens, o.finish_reason) for o in res]
+        for i, o in enumerate(res):
+            assert [t for j, t in seen if j == i] == o.generated_tokens
+        assert eng._inflight is None and not eng.has_work()
+        eng.cache.manager.check()
+        assert eng.cache.manager.live() == []
+        if ahead:
+            assert eng.scheduler.counters["steps"] > 0
+    assert outs[True] == outs[False]
+    assert outs[True][3] == (free[:free.index(free[10]) + 1], "stop")
+    assert [len(t) for t, _ in outs[True]] [:3] == [20, 5, 33] and len(outs[True][4][0]) == 59 + 1 - 50
+
+
 def test_temperature_sampling_is_seeded_and_matches_the_plain_sampler(model_b):
     """Config B's workload: temperature 0.8, 24 tokens, a fixed seed."""
     from deliverance_amd import GeneratorParameters

@@ -182,3 +182,111 @@ def test_random_loads_with_small_pools(seed):
         assert r.finish_reason == FINISH_LENGTH
         assert r.output == expected(r.prompt, r.params.max_tokens)
     assert cache.pools[0].n_free == cache.pools[0].n_pages
+
+
+def drive_ahead(s, cache, max_steps=10000):
+    """As ``drive``, but each step is decided ahead of the one before where the scheduler allows
+    it: the fake model then only learns a request's token when the older step is completed, and a
+    request that ended meanwhile has one step too many, whose result is dropped.  Returns how many
+    steps were decided ahead."""
+    inflight = None          # (batch, sampled tokens by request id), launched but not completed
+    n_ahead = 0
+
+    def launch(batch, prev):
+        sampled = {}
+        for b in batch:
+            if b.samples:
+                toks = b.request.tokens_from(0, min(b.start + b.n, b.request.n_tokens))
+                if b.start + b.n > b.request.n_tokens:         # its last token is the one the older step sampled
+                    toks.append(prev[b.request.rid])
+                sampled[b.request.rid] = fake_next(toks)
+        return batch, sampled
+
+    for _ in range(max_steps):
+        if inflight is not None:
+            nxt = s.schedule_ahead(inflight[0])
+            cache.check()
+            launched = None
+            if nxt is not None:
+                n_ahead += 1
+                assert all(b.n == 1 and b.samples and b.start == b.request.n_tokens for b in nxt)
+                launched = launch(nxt, inflight[1])
+            s.complete(inflight[0], {rid: t for rid, t in inflight[1].items()})
+            cache.check()
+            inflight = launched
+            if inflight is not None:
+                continue
+        if not s.has_work():
+            break
+        batch = s.schedule()
+        cache.check()
+        if batch:
+            assert all(b.start == b.request.n_computed for b in batch)
+            inflight = launch(batch, None)
+    else:
+        raise AssertionError("the scheduler did not come to rest")
+    return n_ahead
+
+
+def test_steps_decided_ahead_give_the_same_tokens():
+    s, cache = make(max_num_seqs=3)
+    a = s.add("a", [1, 2, 3], GeneratorParameters(max_tokens=9))
+    b = s.add("b", [4, 5, 6, 7, 8], GeneratorParameters(max_tokens=4))
+    free = expected([9, 10], 30)
+    s.eos = {free[6]}
+    c = s.add("c", [9, 10], GeneratorParameters(max_tokens=30))
+    n_ahead = drive_ahead(s, cache)
+    assert n_ahead >= 8
+    assert a.output == expected(a.prompt, 9) and a.finish_reason == FINISH_LENGTH
+    assert b.output == expected(b.prompt, 4) and b.finish_reason == FINISH_LENGTH
+    assert c.output == free[:free.index(free[6]) + 1] and c.finish_reason == FINISH_STOP
+    assert cache.pools[0].n_free == cache.pools[0].n_pages and cache.live() == []
+
+
+def test_a_step_is_not_decided_ahead_when_it_could_depend_on_the_tokens():
+    s, cache = make(n_pages=3, page=4, max_num_seqs=2)
+    a = s.add("a", [1, 2, 3], GeneratorParameters(max_tokens=20, ignore_eos=True))
+    batch = s.schedule()
+    # someone waits and a seat is free: admission comes first
+    b = s.add("b", [4, 5], GeneratorParameters(max_tokens=20, ignore_eos=True))
+    assert s.schedule_ahead(batch) is None
+    s.complete(batch, {"a": 5})
+    batch = s.schedule()                       # a decodes, b starts
+    assert {x.request.rid for x in batch} == {"a", "b"}
+    ahead = s.schedule_ahead(batch)            # both at their last token: decided ahead, positions reserved on top
+    assert ahead is not None and [x.start for x in ahead] == [4, 2]
+    s.complete(batch, {"a": 6, "b": 7})
+    s.complete(ahead, {"a": 8, "b": 9})
+    cache.check()
+    # a holds 2 pages (5 positions), b 1 (3 positions): the pool of 3 is spent
+    batch = s.schedule()                       # a at position 5, b at 3: both still fit their pages
+    assert [x.start for x in batch] == [5, 3] and cache.pools[0].n_free == 0
+    # b's position 4 needs a page that is not there: who gives way is decided with the tokens known
+    assert s.schedule_ahead(batch) is None
+    assert cache.length("a") == 5 and cache.length("b") == 3
+    cache.check()
+    s.complete(batch, {"a": 10, "b": 11})
+    batch = s.schedule()
+    # b gave its page back and starts again from its tokens, as far as the one free page reaches
+    assert [(x.request.rid, x.start, x.n) for x in batch] == [("a", 6, 1), ("b", 0, 4)] and b.n_preempted == 1
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_loads_decided_ahead(seed):
+    import random
+    rng = random.Random(100 + seed)
+    s, cache = make(n_pages=rng.randint(8, 14), page=4, max_batch_tokens=rng.choice([6, 12, 32]),
+                    max_chunk=rng.choice([2, 5, 32]), max_num_seqs=rng.randint(1, 4), eos=(5, 6, 7, 8, 9, 10))
+    reqs = []
+    for i in range(10):
+        prompt = [rng.randrange(V) for _ in range(rng.randint(1, 12))]
+        reqs.append(s.add(i, prompt, GeneratorParameters(max_tokens=rng.randint(1, 12))))
+    drive_ahead(s, cache)
+    for r in reqs:
+        want = expected(r.prompt, r.params.max_tokens)
+        stop = next((i for i, t in enumerate(want) if t in s.eos), None)
+        if stop is not None and stop + 1 < len(want):
+            assert r.finish_reason == FINISH_STOP and r.output == want[:stop + 1]
+        else:
+            assert r.output == want
+    assert cache.pools[0].n_free == cache.pools[0].n_pages
