@@ -5,8 +5,8 @@
 // a: [M, K] bf16, w: [N, K] bf16 ("[out, in]", K contiguous), 32-bit accumulation; out is bf16,
 // or 32-bit (plain store or += for the residual stream).  Two kernels:
 //
-//  * gemm_tile: 128x128 block tile, 4 wavefronts of 64x64 (2x2 MFMA 32x32x16), operands staged
-//    through two LDS buffers with the slab after next already in flight.  For steps with many rows
+//  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
+//    buffers, with the next four slabs already in flight in registers.  For steps with many rows
 //    (prefill).
 //  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its
 //    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
@@ -20,7 +20,6 @@
 // row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
 // l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
 #include "gemm_common.h"
-#include <stdlib.h>
 
 #define BKT 64               // k per slab
 #define LDS_LD (BKT + 8)     // padded row length in elements (144 bytes): spreads rows over banks
@@ -32,16 +31,16 @@
 // ---------------------------------------------------------------------------------------------
 // OUTMODE: 0 bf16 store, 1 f32 store, 2 f32 +=.  ACT and OUTMODE are compile-time so that the
 // epilogue is straight-line code.
-template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
-__global__ void __launch_bounds__(WM * WN * 64)
-gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                 Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
+template <int BM, int BN, int WM, int WN, int PF_SLABS, int ACT, int OUTMODE, bool KTAIL>
+__device__ __forceinline__ void
+gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
+               const Epilogue& ep, const KvScatter& kv, int M, int N, int K, int tiles_m, int tiles_n,
+               bf16_t (*As)[BM * LDS_LD], bf16_t (*Ws)[BN * LDS_LD]) {
   constexpr int THREADS = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;       // MFMA tiles per wavefront
   constexpr int CA = BM * 8 / THREADS, CW = BN * 8 / THREADS; // 16-byte chunks per thread and slab
   static_assert(BM * 8 % THREADS == 0 && BN * 8 % THREADS == 0, "tile does not split over the threads");
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_LD];
+  static_assert(PF_SLABS == 2 || PF_SLABS == 4, "two or four slabs in flight");
 
   // Blocks that follow each other in launch order land on different XCDs (8 of them, each with
   // its own L2).  Give each XCD a contiguous run of tiles, m fastest, so that the blocks of one
@@ -68,78 +67,118 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // Loads are never conditional (a conditional load becomes a branch that serialises the slab's
-  // loads): rows past the edge read the last row, chunks past K read chunk 0, and the value is
-  // replaced by zero afterwards.
-  uint4 ra[CA], rw[CW];
+  // loads).  Rows past the edge of a or w read the last row instead: what they produce is never
+  // stored.  Chunks past K (KTAIL: K is no multiple of the slab) read chunk 0 and are replaced by
+  // zero afterwards; that replacement makes the compiler wait for loads early, so it is compiled
+  // only where it is needed.  PF_SLABS slabs are in flight in registers at any time: one slab's
+  // products take far less time than a load, so the distance between asking and needing is what
+  // keeps the matrix cores fed.
+  uint4 ra[PF_SLABS][CA], rw[PF_SLABS][CW];
   const uint4 zero = make_uint4(0, 0, 0, 0);
   const bf16_t* pa[CA];
   const bf16_t* pw[CW];
-  bool oka[CA], okw[CW];
 #pragma unroll
   for (int i = 0; i < CA; ++i) {
     const int c = t + THREADS * i, row = m0 + c / 8;
-    oka[i] = row < M;
-    pa[i] = a + (size_t)(oka[i] ? row : M - 1) * lda + (c % 8) * 8;
+    pa[i] = a + (size_t)(row < M ? row : M - 1) * lda + (c % 8) * 8;
   }
 #pragma unroll
   for (int i = 0; i < CW; ++i) {
     const int c = t + THREADS * i, row = n0 + c / 8;
-    okw[i] = row < N;
-    pw[i] = w + (size_t)(okw[i] ? row : N - 1) * ldw + (c % 8) * 8;
+    pw[i] = w + (size_t)(row < N ? row : N - 1) * ldw + (c % 8) * 8;
   }
   const int kc_t = (t % 8) * 8;                     // this thread's chunk offset inside a slab (THREADS % 8 == 0)
-  auto fetch = [&](int k0) {
-    const bool kin = k0 + kc_t < K;
-    const int ks = kin ? k0 : 0;
-#pragma unroll
-    for (int i = 0; i < CA; ++i) {
-      ra[i] = load16(pa[i] + ks);
-      if (!(kin && oka[i])) ra[i] = zero;
-    }
-#pragma unroll
-    for (int i = 0; i < CW; ++i) {
-      rw[i] = load16(pw[i] + ks);
-      if (!(kin && okw[i])) rw[i] = zero;
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < CA; ++i) {
-      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;
-      *(uint4*)&As[buf][row * LDS_LD + kc] = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < CW; ++i) {
-      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;
-      *(uint4*)&Ws[buf][row * LDS_LD + kc] = rw[i];
-    }
-  };
+#define TILE_FETCH(stage, k0)                                   \
+  {                                                             \
+    const bool kin = !KTAIL || (k0) + kc_t < K;                 \
+    const int ks = kin ? (k0) : 0;                              \
+    _Pragma("unroll") for (int i = 0; i < CA; ++i) {            \
+      ra[stage][i] = load16(pa[i] + ks);                        \
+      if (KTAIL && !kin) ra[stage][i] = zero;                   \
+    }                                                           \
+    _Pragma("unroll") for (int i = 0; i < CW; ++i) {            \
+      rw[stage][i] = load16(pw[i] + ks);                        \
+      if (KTAIL && !kin) rw[stage][i] = zero;                   \
+    }                                                           \
+  }
+#define TILE_STASH(stage, buf)                                              \
+  {                                                                         \
+    _Pragma("unroll") for (int i = 0; i < CA; ++i) {                        \
+      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;         \
+      *(uint4*)&As[buf][row * LDS_LD + kc] = ra[stage][i];                  \
+    }                                                                       \
+    _Pragma("unroll") for (int i = 0; i < CW; ++i) {                        \
+      const int c = t + THREADS * i, row = c / 8, kc = (c % 8) * 8;         \
+      *(uint4*)&Ws[buf][row * LDS_LD + kc] = rw[stage][i];                  \
+    }                                                                       \
+  }
   const int fr = lane % 32, fk = (lane / 32) * 8;
   const int nslab = (K + BKT - 1) / BKT;
-  fetch(0);
-  stash(0);
-  lds_barrier();
-  for (int sidx = 0; sidx < nslab; ++sidx) {
-    const int buf = sidx & 1;
-    if (sidx + 1 < nslab) fetch((sidx + 1) * BKT);      // in flight while this slab is multiplied
+  // what the output held before (+=) is asked for now, from clamped places, and has long arrived
+  // when the products are done
+  float old[OUTMODE == 2 ? TM : 1][OUTMODE == 2 ? TN : 1][OUTMODE == 2 ? 16 : 1];
+  if (OUTMODE == 2) {
 #pragma unroll
-    for (int kk = 0; kk < BKT; kk += 16) {
-      bf16x8_t af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        af[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&As[buf][(wm + i * 32 + fr) * LDS_LD + kk + fk]);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bf[j] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ws[buf][(wn + j * 32 + fr) * LDS_LD + kk + fk]);
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn + j * 32 + fr, nc = n < N ? n : N - 1;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4), mc = m < M ? m : M - 1;
+          old[OUTMODE == 2 ? i : 0][OUTMODE == 2 ? j : 0][OUTMODE == 2 ? r : 0] =
+              ((const float*)ep.out)[(size_t)mc * ep.ldo + nc];
+        }
     }
-    if (sidx + 1 < nslab) stash(buf ^ 1);               // the other buffer was last read before the previous barrier
-    lds_barrier();
   }
+#pragma unroll
+  for (int j = 0; j < PF_SLABS; ++j)
+    if (j < nslab) TILE_FETCH(j, j * BKT);
+  TILE_STASH(0, 0);
+  lds_barrier();
+  // One slab: stage j's registers went to LDS before the last barrier and take the slab PF_SLABS
+  // further on; the products of slab sidx come out of LDS buffer j & 1 (= sidx & 1, PF_SLABS is
+  // even); the next slab's registers go to the other buffer, which was last read before the
+  // previous barrier.
+#define TILE_STEP(j, sidx, want_fetch, want_stash)                                                              \
+  {                                                                                                             \
+    constexpr int buf = (j) & 1;                                                                                \
+    if (want_fetch) TILE_FETCH(j, ((sidx) + PF_SLABS) * BKT);                                                   \
+    _Pragma("unroll") for (int kk = 0; kk < BKT; kk += 16) {                                                    \
+      bf16x8_t af[TM], bf[TN];                                                                                  \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                            \
+        af[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&As[buf][(wm + i * 32 + fr) * LDS_LD + kk + fk]);   \
+      _Pragma("unroll") for (int jj = 0; jj < TN; ++jj)                                                         \
+        bf[jj] = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ws[buf][(wn + jj * 32 + fr) * LDS_LD + kk + fk]); \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                            \
+        _Pragma("unroll") for (int jj = 0; jj < TN; ++jj)                                                       \
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[jj], acc[i][jj], 0, 0, 0);             \
+    }                                                                                                           \
+    if (want_stash) TILE_STASH(((j) + 1) % PF_SLABS, buf ^ 1);                                                  \
+    lds_barrier();                                                                                              \
+  }
+  // The steady state has no branches, so that the compiler counts the loads in flight exactly and
+  // waits for the oldest slab only; the last slabs run through the same steps with conditions.
+  int base = 0;
+  for (; base + 2 * PF_SLABS <= nslab; base += PF_SLABS) {
+    TILE_STEP(0, base, true, true);
+    TILE_STEP(1, base + 1, true, true);
+    if (PF_SLABS == 4) {
+      TILE_STEP(2, base + 2, true, true);
+      TILE_STEP(3, base + 3, true, true);
+    }
+  }
+  for (; base < nslab; base += PF_SLABS) {
+    if (base < nslab) TILE_STEP(0, base, base + PF_SLABS < nslab, base + 1 < nslab);
+    if (base + 1 < nslab) TILE_STEP(1, base + 1, base + 1 + PF_SLABS < nslab, base + 2 < nslab);
+    if (PF_SLABS == 4) {
+      if (base + 2 < nslab) TILE_STEP(2, base + 2, base + 2 + PF_SLABS < nslab, base + 3 < nslab);
+      if (base + 3 < nslab) TILE_STEP(3, base + 3, base + 3 + PF_SLABS < nslab, base + 4 < nslab);
+    }
+  }
+#undef TILE_STEP
+#undef TILE_FETCH
+#undef TILE_STASH
 
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -154,7 +193,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
         if (m < M) {
           const float v = apply_act(acc[i][j][r] + b, ACT);
           const size_t o = (size_t)m * ep.ldo + n;
-          if (OUTMODE == 2) ((float*)ep.out)[o] += v;
+          if (OUTMODE == 2) ((float*)ep.out)[o] = old[OUTMODE == 2 ? i : 0][OUTMODE == 2 ? j : 0][OUTMODE == 2 ? r : 0] + v;
           else if (OUTMODE == 1) ((float*)ep.out)[o] = v;
           else ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
           if (OUTMODE == 0 && kv.cache && n >= kv.q_cols) {
@@ -166,28 +205,38 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
   }
 }
 
-template <int BM, int BN, int WM, int WN, int ACT>
+template <int BM, int BN, int WM, int WN, int PF, int ACT, int OUTMODE>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
+                 Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_LD];      // shared by the two bodies
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_LD];
+  if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, As, Ws);
+  else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, As, Ws);
+}
+
+template <int BM, int BN, int WM, int WN, int PF, int ACT>
 static void launch_tile_act(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
                             const KvScatter& kv, int M, int N, int K) {
   const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
   const dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if (ep.accumulate)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else if (ep.out_dtype == DA_F32)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int PF>
 static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
                         const KvScatter& kv, int M, int N, int K) {
   switch (ep.act) {
-    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    default: launch_tile_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    default: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
   }
 }
 
@@ -309,22 +358,19 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     dim3 grid(da_ceil_div(N, SK_COLS));
     const int mt = da_ceil_div(M, 16);
     // the number of wavefronts that split K depends on K alone, so a row's sums keep their order
-    static int force_nw = -1;
-    if (force_nw < 0) { const char* e = getenv("DA_SKINNY_NW"); force_nw = e ? atoi(e) : 0; }
-    int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
-    if (force_nw > 0) nw = force_nw;
+    const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
     if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
     else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else if (nw == 4) launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else launch_skinny<2>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
   } else {
-    // Smaller tiles where 128x128 tiles would leave compute units idle.  Every configuration sums a
-    // row's products in the same order (64-wide slabs, 16 at a time), so the choice does not change
-    // a result.
+    // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
+    // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so
+    // the choice does not change a result.
     const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
-    if (tiles128 < 128) launch_tile<64, 64, 2, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
-    else if (tiles128 < 256) launch_tile<128, 64, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
-    else launch_tile<128, 128, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+    const long tiles12864 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 64);
+    if (tiles128 >= 192) launch_tile<128, 128, 4, 2, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+    else if (tiles12864 >= 192) launch_tile<128, 64, 4, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
+    else launch_tile<64, 64, 2, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
   }
   DA_CHECK_LAUNCH("gemm_bf16");
   return 0;
