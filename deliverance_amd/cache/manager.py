@@ -21,6 +21,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 
 class CacheError(RuntimeError):
     """Misuse of the cache manager (unknown request, double free, ...)."""
@@ -237,6 +239,13 @@ class CacheManager:
         """Cache row (page * page_size + offset) of positions start .. start+n-1."""
         t = self._req(rid).tables[group]
         ps = self.page_size
+        if n > 16:                                   # long portions: the same by arrays
+            pos = np.arange(start, start + n, dtype=np.int64)
+            pages = np.asarray(t, dtype=np.int64)[pos // ps]
+            if (pages < 0).any():
+                p = int(pos[pages < 0][0])
+                raise CacheError(f"position {p} of {rid!r} lies in a page that was given back")
+            return (pages * ps + pos % ps).tolist()
         out = []
         for p in range(start, start + n):
             page = t[p // ps]

@@ -13,11 +13,13 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import OutOfPages
 from ..models.causal_lm import CausalLM
 from ..parts.base import Arena, StepContext
+from ..sampling.sampler import RECORD_WORDS
 from .device_cache import DeviceCache
 
 
@@ -54,16 +56,19 @@ class StepRunner:
         self.sampled = torch.zeros(2 * max(64, max_graph_batch), dtype=torch.int32, device=self.device)
 
     # ---- host -> device in one copy --------------------------------------------------------
-    def _upload(self, words: List[int]) -> torch.Tensor:
-        n = len(words)
+    def _staging_for(self, n: int):
+        """The pinned buffer (as a numpy view) that the step's ``n`` integers are written into."""
         if self._staging is None or self._staging.numel() < n:
             cap = max(4096, 2 * n)
             self._staging = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._staging_np = self._staging.numpy()
             self._staging_dev = torch.empty(cap, dtype=torch.int32, device=self.device)
             self._copied = None
         if self._copied is not None:
             self._copied.synchronize()       # the last step's copy has read the pinned buffer
-        self._staging[:n] = torch.tensor(words, dtype=torch.int32)
+        return self._staging_np[:n]
+
+    def _upload(self, n: int) -> torch.Tensor:
         self._staging_dev[:n].copy_(self._staging[:n], non_blocking=True)
         self._copied = torch.cuda.Event()
         self._copied.record()
@@ -90,9 +95,13 @@ class StepRunner:
             seen.add(e.rid)
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.rid!r} brings no tokens")
-            for t in e.tokens:
-                if not (0 <= int(t) < cfg.vocab_size):
-                    raise StepError(f"request {e.rid!r}: token id {t} is outside the vocabulary of {cfg.vocab_size}")
+            if len(e.tokens) <= 8:
+                bad = [t for t in e.tokens if not (0 <= int(t) < cfg.vocab_size)]
+            else:
+                arr = np.asarray(e.tokens, dtype=np.int64)
+                bad = arr[(arr < 0) | (arr >= cfg.vocab_size)].tolist()
+            if bad:
+                raise StepError(f"request {e.rid!r}: token id {bad[0]} is outside the vocabulary of {cfg.vocab_size}")
             for w in e.want:
                 if not (0 <= int(w) < len(e.tokens)):
                     raise StepError(f"request {e.rid!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
@@ -137,9 +146,9 @@ class StepRunner:
                     mgr.commit(e.rid)
             return logits, ctx
 
-        words, offs, meta = self._pack(entries, order, starts, pad_to=None, max_blocks=None,
-                                       extra=sample_records)
-        dev = self._upload(words)
+        offs, meta, n_words = self._layout(entries, order, pad_to=None, max_blocks=None, extra=sample_records)
+        self._fill(self._staging_for(n_words), offs, meta, entries, order, starts, sample_records)
+        dev = self._upload(n_words)
         ctx = self._context(dev, offs, meta, self.arena)
         self.last_ctx = ctx
         R = meta["R"]
@@ -153,43 +162,22 @@ class StepRunner:
         return logits, ctx
 
     # ---- packing the step's integers -----------------------------------------------------------
-    def _pack(self, entries, order, starts, pad_to, max_blocks, extra):
-        """All integers of a step in one list: tokens, positions, sequence ids, row starts, lengths,
-        state slots, wanted rows, then per cache group the cache row of every token and the block
-        tables, then ``extra``.  With ``pad_to`` the step is filled up with empty one-token
-        sequences (length 0, no cache row), so that its shape is fixed."""
+    def _layout(self, entries, order, pad_to, max_blocks, extra):
+        """Where each array of the step lies in its one buffer of integers: tokens, where a token
+        comes from, positions, sequence ids, row starts, lengths, state slots, wanted rows, then
+        per cache group the cache row of every token and the block tables, then ``extra``.  With
+        ``pad_to`` the step is filled up with empty one-token sequences (length 0, no cache row),
+        so that its shape is fixed."""
         mgr = self.cache.manager
         S_real = len(entries)
-        tokens: List[int] = []
-        token_src: List[int] = []
-        positions: List[int] = []
-        seq_of: List[int] = []
-        q_start = [0]
-        seq_lens: List[int] = []
-        state_slots: List[int] = []
-        row0 = {}
-        for s, i in enumerate(order):
-            e = entries[i]
-            st = starts[e.rid]
-            row0[i] = len(tokens)
-            tokens += [int(t) for t in e.tokens]
-            token_src += [e.from_sampled] if e.from_sampled is not None else [-1] * len(e.tokens)
-            positions += list(range(st, st + len(e.tokens)))
-            seq_of += [s] * len(e.tokens)
-            q_start.append(len(tokens))
-            seq_lens.append(st + len(e.tokens))
-            state_slots.append(mgr.state_slot(e.rid))
-        want_rows = [row0[i] + int(w) for i, e in enumerate(entries) for w in e.want]
         n_pad = 0 if pad_to is None else pad_to - S_real
-        for k in range(n_pad):
-            tokens.append(0); token_src.append(-1); positions.append(0); seq_of.append(S_real + k)
-            q_start.append(len(tokens)); seq_lens.append(0); state_slots.append(-1)
-            want_rows.append(len(tokens) - 1)
-        N, S, R = len(tokens), S_real + n_pad, len(want_rows)
+        N = sum(len(e.tokens) for e in entries) + n_pad
+        S = S_real + n_pad
+        R = sum(len(e.want) for e in entries) + n_pad
         G = len(self.cache.groups)
         if max_blocks is None:
-            max_blocks = max(1, max(len(mgr.table(entries[i].rid, g)) for i in order for g in range(G))) if G else 1
-        words = tokens + token_src + positions + seq_of + q_start + seq_lens + state_slots + want_rows
+            max_blocks = max(1, max(len(mgr.table(e.rid, g)) for e in entries for g in range(G))) if G else 1
+        n_extra = 0 if not extra else len(extra) + RECORD_WORDS * n_pad
         offs = {}
         o = 0
         for name, n in (("tokens", N), ("token_src", N), ("positions", N), ("seq_of", N), ("q_start", S + 1),
@@ -197,26 +185,86 @@ class StepRunner:
             offs[name] = (o, n)
             o += n
         for g in range(G):
-            sm: List[int] = []
-            bt: List[int] = []
-            for i in order:
-                e = entries[i]
-                sm += mgr.slots_for(e.rid, g, starts[e.rid], len(e.tokens))
-                t = mgr.table(e.rid, g)
-                bt += t + [-1] * (max_blocks - len(t))
-            sm += [-1] * n_pad
-            bt += [-1] * (n_pad * max_blocks)
-            words += sm + bt
             offs[f"slot_map{g}"] = (o, N)
             offs[f"block_table{g}"] = (o + N, S * max_blocks)
             o += N + S * max_blocks
-        if extra:
-            extra = list(extra) + [0] * (8 * n_pad if pad_to is not None else 0)
-            words += extra
-            offs["extra"] = (o, len(extra))
-        meta = dict(N=N, S=S, R=R, G=G, max_blocks=max_blocks, n_decode=sum(1 for e in entries if len(e.tokens) == 1) + n_pad,
-                    q_start=q_start, seq_lens=seq_lens, state_slots=state_slots)
-        return words, offs, meta
+        if n_extra:
+            offs["extra"] = (o, n_extra)
+            o += n_extra
+        meta = dict(N=N, S=S, R=R, G=G, max_blocks=max_blocks, n_pad=n_pad,
+                    n_decode=sum(1 for e in entries if len(e.tokens) == 1) + n_pad)
+        return offs, meta, o
+
+    def _fill(self, buf, offs, meta, entries, order, starts, extra):
+        """Write the step's integers into ``buf`` (a numpy view of pinned memory).  Long portions
+        are written as arrays, single tokens as scalars."""
+        mgr = self.cache.manager
+        ps = self.cache.page_size
+
+        def view(name):
+            a, n = offs[name]
+            return buf[a:a + n]
+        tok, src, pos, seq = view("tokens"), view("token_src"), view("positions"), view("seq_of")
+        q_start_v, seq_lens_v, state_v, want_v = view("q_start"), view("seq_lens"), view("state_slots"), view("want")
+        G, mb, n_pad = meta["G"], meta["max_blocks"], meta["n_pad"]
+        sms = [view(f"slot_map{g}") for g in range(G)]
+        bts = [view(f"block_table{g}") for g in range(G)]
+        for bt in bts:
+            bt[:] = -1
+        q_start, seq_lens, state_slots = [0], [], []
+        row0 = {}
+        row = 0
+        for s, i in enumerate(order):
+            e = entries[i]
+            n = len(e.tokens)
+            st = starts[e.rid]
+            row0[i] = row
+            if n == 1:
+                tok[row] = e.tokens[0]
+                src[row] = -1 if e.from_sampled is None else e.from_sampled
+                pos[row] = st
+                seq[row] = s
+            else:
+                tok[row:row + n] = e.tokens
+                src[row:row + n] = -1
+                pos[row:row + n] = np.arange(st, st + n, dtype=np.int32)
+                seq[row:row + n] = s
+            for g in range(G):
+                t = mgr.table(e.rid, g)
+                if n == 1:
+                    page = t[st // ps]
+                    if page < 0:
+                        raise StepError(f"position {st} of {e.rid!r} lies in a page that was given back")
+                    sms[g][row] = page * ps + st % ps
+                else:
+                    sms[g][row:row + n] = mgr.slots_for(e.rid, g, st, n)
+                bts[g][s * mb:s * mb + len(t)] = t
+            row += n
+            q_start.append(row)
+            seq_lens.append(st + n)
+            state_slots.append(mgr.state_slot(e.rid))
+        S_real = len(entries)
+        r = 0
+        for i, e in enumerate(entries):
+            for w in e.want:
+                want_v[r] = row0[i] + int(w)
+                r += 1
+        for k in range(n_pad):          # empty one-token sequences
+            tok[row] = 0; src[row] = -1; pos[row] = 0; seq[row] = S_real + k
+            for g in range(G):
+                sms[g][row] = -1
+            want_v[r] = row
+            r += 1
+            row += 1
+            q_start.append(row); seq_lens.append(0); state_slots.append(-1)
+        q_start_v[:] = q_start
+        seq_lens_v[:] = seq_lens
+        state_v[:] = state_slots
+        if "extra" in offs:
+            ex = view("extra")
+            ex[:len(extra)] = extra
+            ex[len(extra):] = 0
+        meta.update(q_start=q_start, seq_lens=seq_lens, state_slots=state_slots)
 
     def _context(self, dev, offs, meta, arena) -> StepContext:
         def view(name):
@@ -252,18 +300,19 @@ class StepRunner:
         while bucket < S:
             bucket *= 2
         order = list(range(S))
-        words, offs, meta = self._pack(entries, order, starts, pad_to=bucket, max_blocks=self.max_blocks_cap,
-                                       extra=sample_records)
+        offs, meta, n_words = self._layout(entries, order, pad_to=bucket, max_blocks=self.max_blocks_cap,
+                                           extra=sample_records)
         st = self._graphs.get(bucket)
         if st is None:
-            st = {"dev": torch.empty(len(words), dtype=torch.int32, device=self.device),
-                  "host": torch.empty(len(words), dtype=torch.int32, pin_memory=True),
+            host = torch.empty(n_words, dtype=torch.int32, pin_memory=True)
+            st = {"dev": torch.empty(n_words, dtype=torch.int32, device=self.device),
+                  "host": host, "host_np": host.numpy(),
                   "arena": Arena(self.device), "graph": None, "copied": None}
             self._graphs[bucket] = st
-        assert st["dev"].numel() == len(words), "a bucket's layout is fixed"
+        assert st["dev"].numel() == n_words, "a bucket's layout is fixed"
         if st["copied"] is not None:
             st["copied"].synchronize()
-        st["host"].copy_(torch.tensor(words, dtype=torch.int32))
+        self._fill(st["host_np"], offs, meta, entries, order, starts, sample_records)
         st["dev"].copy_(st["host"], non_blocking=True)
         st["copied"] = torch.cuda.Event()
         st["copied"].record()
