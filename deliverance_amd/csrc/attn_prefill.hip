@@ -4,7 +4,7 @@
 // written just before).
 //
 // One workgroup per (portion, query head, 32 * W query rows); W wavefronts of 32 rows each.  Keys
-// come in aligned tiles of 64 through LDS: the key rows as they lie in the pages, the values as
+// come in aligned tiles of 64 through two LDS buffers, two tiles ahead in registers: the key rows as they lie in the pages, the values as
 // they lie in the pages too (dimension-major: a row of the LDS tile is one dimension, 64 keys).
 // Per tile and wavefront, with MFMA 32x32x16:
 //   S^T[key, row] = K . Q^T          keys are the MFMA's rows, so one lane holds ONE query row's
@@ -18,7 +18,6 @@
 // A row's sums run over key tiles in ascending order starting at the aligned tile of its lo: the
 // order depends on the row's position (and window) only.
 #include "common.h"
-#include <stdlib.h>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
@@ -27,7 +26,10 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 #define PF_VLD (PF_BK + 8) // padded length of a value row in LDS
 #define PF_BT_MAX 2048      // block-table entries a workgroup keeps in LDS (more are read from memory)
 
-template <int D16, int PF_WAVES>   // head size / 16; wavefronts (32 query rows each) per workgroup
+// head size / 16; wavefronts (32 query rows each) per workgroup; whether the block table's entries
+// for the workgroup's keys fit its LDS copy (a table entry read from memory in front of a tile's loads
+// makes them wait for it, and for every load still in flight)
+template <int D16, int PF_WAVES, bool BT_LDS>
 __global__ void __launch_bounds__(PF_WAVES * DA_WAVE)
 attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                     const int* __restrict__ block_table, int max_blocks,
@@ -41,13 +43,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   constexpr int THREADS = PF_WAVES * DA_WAVE;
   constexpr int K_PIECES = PF_BK * (D / 8), V_PIECES = DT * 32 * (PF_BK / 8);   // 16-byte pieces of a tile
   constexpr int NK = (K_PIECES + THREADS - 1) / THREADS, NV = (V_PIECES + THREADS - 1) / THREADS;  // per thread
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BK * KLD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[DT * 32 * PF_VLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][PF_BK * KLD];          // a tile is multiplied out of one
+  __shared__ __attribute__((aligned(16))) bf16_t Vs2[2][DT * 32 * PF_VLD];     // while the next is parked in the other
   __shared__ int bts[PF_BT_MAX];
 
   const int s = seq0 + blockIdx.z, h = blockIdx.y;
   const int row0 = q_start[s], T = q_start[s + 1] - row0;
-  const int i0 = blockIdx.x * PF_BQ;
+  // the workgroups with the most keys (the last rows) are launched first
+  const int i0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * PF_BQ;
   if (i0 >= T) return;
   const int past = seq_lens[s] - T;
   const int hk = h / (Hq / Hkv);
@@ -93,17 +96,32 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   // from memory in front of every tile would make the tile's loads wait for it, and that wait also
   // drains the loads still in flight for the tiles before.
   const int pg_lo = b_lo >> (31 - __builtin_clz(page)), pg_hi = b_last >> (31 - __builtin_clz(page));
-  const bool bt_local = pg_hi - pg_lo + 1 <= PF_BT_MAX;
-  if (bt_local)
+  if (BT_LDS)
     for (int i = t; i <= pg_hi - pg_lo; i += THREADS) bts[i] = bt[pg_lo + i];
   __syncthreads();
-  auto page_of = [&](int key_page) -> long long { return bt_local ? bts[key_page - pg_lo] : bt[key_page]; };
+  auto page_of = [&](int key_page) -> long long { return BT_LDS ? bts[key_page - pg_lo] : bt[key_page]; };
   // Two register sets: while a tile is multiplied, the loads of the next two are in flight.
   uint4 rk0[NK], rv0[NV], rk1[NK], rv1[NV];
   const int lg = 31 - __builtin_clz(page);              // page is a power of two (checked on the host)
   const long long page_elems = 2LL * Hkv * page * D;
   const bf16_t* kbase = cache + (long long)hk * page * D;
   const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
+  // a tile whose 64 keys all lie in b_lo .. b_last: nothing to clamp, nothing to replace
+  auto fetch_fast = [&](uint4* rk, uint4* rv, int kt) {
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int c0 = t + i * THREADS, c = c0 < K_PIECES ? c0 : 0;
+      const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
+      rk[i] = *(const uint4*)(kbase + page_of(key >> lg) * page_elems + (key & (page - 1)) * D + pc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
+      const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;
+      const int ds = d < D ? d : 0;                      // rows of a padded 32-dimension tile repeat dimension 0
+      rv[i] = *(const uint4*)(vbase + page_of(key0 >> lg) * page_elems + ds * page + (key0 & (page - 1)));
+    }
+  };
   auto fetch = [&](uint4* rk, uint4* rv, int kt) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
@@ -133,34 +151,26 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       rv[i] = v;
     }
   };
-  auto stash = [&](const uint4* rk, const uint4* rv) {
+  auto stash = [&](const uint4* rk, const uint4* rv, int buf) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int c = t + i * THREADS, kr = c / (D / 8), pc = c % (D / 8);
-      if (c < K_PIECES) *(uint4*)&Ks[kr * KLD + pc * 8] = rk[i];
+      if (K_PIECES % THREADS == 0 || c < K_PIECES) *(uint4*)&Ks2[buf][kr * KLD + pc * 8] = rk[i];
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = t + i * THREADS, d = c / (PF_BK / 8), g = c % (PF_BK / 8);
-      if (c < V_PIECES) *(uint4*)&Vs[d * PF_VLD + g * 8] = rv[i];
+      if (V_PIECES % THREADS == 0 || c < V_PIECES) *(uint4*)&Vs2[buf][d * PF_VLD + g * 8] = rv[i];
     }
   };
   const int kt0 = (b_lo / PF_BK) * PF_BK;
   fetch(rk0, rv0, kt0);
   if (kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
-  int parity = 0;
-  for (int kt = kt0; kt <= b_last; kt += PF_BK, parity ^= 1) {
-    // this tile's registers go to LDS; the set is then free for the tile after next
-    if (parity == 0) {
-      stash(rk0, rv0);
-      lds_barrier();
-      if (kt + 2 * PF_BK <= b_last) fetch(rk0, rv0, kt + 2 * PF_BK);
-    } else {
-      stash(rk1, rv1);
-      lds_barrier();
-      if (kt + 2 * PF_BK <= b_last) fetch(rk1, rv1, kt + 2 * PF_BK);
-    }
 
+  // the products of one tile, out of LDS buffer `buf`
+  auto tile = [&](int kt, int buf) {
+    const bf16_t* Ks = Ks2[buf];
+    const bf16_t* Vs = Vs2[buf];
     if (wave_on && kt <= w_last && kt + PF_BK - 1 >= w_lo) {
       floatx16 sc[2];
 #pragma unroll
@@ -173,32 +183,35 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           sc[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kd], sc[ks], 0, 0, 0);
         }
       }
-      // Scale, mask, running maximum and weights.  Scores are kept in the base-2 domain
-      // (s * scale * log2 e), so that a weight costs one subtraction and one hardware exp2.  A tile
-      // that every row of the wavefront sees whole needs no mask at all.
+      // Mask, running maximum and weights.  The maximum is kept in the base-2 domain
+      // (s * scale * log2 e, scale > 0), so that a weight costs one multiply-add and one hardware
+      // exp2.  A tile that every row of the wavefront sees whole needs no mask at all; elsewhere a key
+      // outside q_lo .. pq gets -inf added (0 otherwise), computed from the sign of
+      // min(pq - key, key - q_lo) without a comparison: scores are finite, keys that do not exist
+      // were loaded as zeros.
       const bool whole = kt + PF_BK - 1 <= w_first && (window <= 0 || kt >= w_last - window + 1);
       float tmax = -INFINITY;
       if (whole) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            sc[ks][r] *= scale2;
-            tmax = fmaxf(tmax, sc[ks][r]);
-          }
+          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sc[ks][r]);
       } else {
+        const int d0 = (q_ok ? pq : -(1 << 30)) - kt - 4 * hf;      // pq - key for the lane's first key
+        const int e0 = (pq - q_lo) - d0;                             // key - q_lo likewise
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int key = kt + ks * 32 + 8 * (r / 4) + 4 * hf + (r % 4);
-            const bool vis = q_ok && key <= pq && key >= q_lo;
-            const float v = vis ? sc[ks][r] * scale2 : -INFINITY;
+            const int c = ks * 32 + 8 * (r / 4) + (r % 4);
+            const int lo = min(d0 - c, e0 + c);
+            const float bias = __builtin_bit_cast(float, (lo >> 31) & (int)0xff800000);
+            const float v = sc[ks][r] + bias;
             sc[ks][r] = v;
             tmax = fmaxf(tmax, v);
           }
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DA_WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DA_WAVE)) * scale2;
       const float m_new = fmaxf(m, tmax);
       const bool any = m_new != -INFINITY;             // a row that has seen no key yet keeps zeros
       const float m_use = any ? m_new : 0.f;           // -inf - 0 stays -inf: weight 0, never NaN
@@ -212,8 +225,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           uint32_t u[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float p0 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e] - m_use);
-            const float p1 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e + 1] - m_use);
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[ks][kb * 8 + 2 * e], scale2, -m_use));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[ks][kb * 8 + 2 * e + 1], scale2, -m_use));
             tsum += p0 + p1;
             u[e] = pack2_bf16(p0, p1);
           }
@@ -222,6 +235,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       tsum += __shfl_xor(tsum, 32, DA_WAVE);
       l = l * alpha + tsum;
       m = m_new;
+      // (skipping this when no row's maximum rose costs a second copy of the output's registers at
+      // the branch, and with it half of the wavefronts a compute unit holds)
 #pragma unroll
       for (int i = 0; i < DT; ++i)
 #pragma unroll
@@ -239,7 +254,35 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[ks][kb], acc_o[i], 0, 0, 0);
           }
     }
+  };
+
+  // Steady state, two tiles a round, without a branch around the loads: the compiler then counts the
+  // loads in flight exactly and a tile waits for its own registers only.  It lasts while the tile
+  // asked for (two ahead) lies whole inside the workgroup's keys; the last tiles run through the
+  // same steps with conditions and the clamping loads.  One barrier a tile: the buffer written now
+  // was last read two tiles ago, before the previous barrier.
+  int kt = kt0;
+  for (; kt + 4 * PF_BK - 1 <= b_last; kt += 2 * PF_BK) {
+    stash(rk0, rv0, 0);
     lds_barrier();
+    fetch_fast(rk0, rv0, kt + 2 * PF_BK);
+    tile(kt, 0);
+    stash(rk1, rv1, 1);
+    lds_barrier();
+    fetch_fast(rk1, rv1, kt + 3 * PF_BK);
+    tile(kt + PF_BK, 1);
+  }
+  for (int parity = 0; kt <= b_last; kt += PF_BK, parity ^= 1) {
+    if (parity == 0) {
+      stash(rk0, rv0, 0);
+      lds_barrier();
+      if (kt + 2 * PF_BK <= b_last) fetch(rk0, rv0, kt + 2 * PF_BK);
+    } else {
+      stash(rk1, rv1, 1);
+      lds_barrier();
+      if (kt + 2 * PF_BK <= b_last) fetch(rk1, rv1, kt + 2 * PF_BK);
+    }
+    tile(kt, parity);
   }
 
   if (q_ok) {
@@ -271,17 +314,20 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   DA_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)cache % 16 == 0) && ((uintptr_t)out % 8 == 0),
              "attn_prefill: operands must be 16-byte aligned");
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_prefill: bad window or block table");
+  DA_REQUIRE(scale > 0.f, "attn_prefill: the score scale must be positive, found %g", (double)scale);
   DA_REQUIRE(n_seqs <= 65535 && Hq <= 65535, "attn_prefill: too many sequences or heads for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
-  const int waves = 4;
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH2(N, W)                                                                                     \
-  hipLaunchKernelGGL((attn_prefill_kernel<N, W>), dim3(da_ceil_div(max_query_len, 32 * W), Hq, n_seqs),   \
+  // every key a workgroup can see lies within max_blocks pages
+  const bool bt_lds = max_blocks <= PF_BT_MAX;
+#define LAUNCH2(N, W, L)                                                                                  \
+  hipLaunchKernelGGL((attn_prefill_kernel<N, W, L>), dim3(da_ceil_div(max_query_len, 32 * W), Hq, n_seqs), \
                      dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
                      max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld)
-#define LAUNCH(N)        \
-  case N:                \
-    LAUNCH2(N, 4);       \
+#define LAUNCH(N)                      \
+  case N:                              \
+    if (bt_lds) LAUNCH2(N, 4, true);   \
+    else LAUNCH2(N, 4, false);         \
     break;
   switch (D / 16) {
     LAUNCH(1) LAUNCH(2) LAUNCH(3) LAUNCH(4) LAUNCH(5) LAUNCH(6) LAUNCH(7) LAUNCH(8)

@@ -26,6 +26,10 @@ ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-result", "-Wno-unknown-warning-option"]
+# Per source: kernels that read their matrix-core results back at once (softmax between two
+# products) keep them in ordinary vector registers; the default puts them into accumulation
+# registers and moves every value out and in again.
+EXTRA_FLAGS = {"attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _lib = None
 
@@ -115,7 +119,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
 
     def compile_one(src):
         obj = os.path.join(out_dir, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(os.path.basename(src), []), "-I", CSRC, "-c", src, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True, env=env)
         if r.returncode != 0:
             raise KernelLibraryError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
