@@ -6,12 +6,15 @@
 //
 // `w` is [N, K] with K contiguous ("[out, in]"), the layout the reference multiplies against
 // (tensor/src/main/java/io/teknek/deliverance/tensor/operations/NaiveTensorOperations.java:86-91).
-// Every output element sums over k in ascending order, whatever M is, so a row's result does
-// not depend on which other rows share the step.
+// Every output element sums over k in the same order, whatever M is, so a row's result does
+// not depend on which other rows share the step: products are summed in ascending order within
+// chunks of 128, and the chunks' sums are added in ascending order (a long sum into one 32-bit
+// accumulator loses about sqrt(K) roundings; in two levels it loses sqrt(128) + sqrt(K / 128)).
 #include "common.h"
 
 #define TILE 64
 #define BK 16
+#define CHUNK_SLABS 8      // slabs of BK that are summed before their sum joins the total
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -24,12 +27,13 @@ gemm_ref_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, int l
   const int tx = t % 16, ty = t / 16;
   const int m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE;
   const int lrow = t / 4, lk = (t % 4) * 4;
-  float acc[4][4];
+  float acc[4][4], part[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = part[i][j] = 0.f;
 
+  int slab = 0;
   for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -49,10 +53,24 @@ gemm_ref_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, int l
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(av[i], wv[j], part[i][j]);
+    }
+    if (++slab == CHUNK_SLABS) {
+      slab = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] += part[i][j];
+          part[i][j] = 0.f;
+        }
     }
     __syncthreads();
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;

@@ -109,12 +109,16 @@ __device__ __forceinline__ float4 load_param4(const void* p, int dtype, int i) {
 
 // The same norm with the whole row held in registers: every load of the row is in flight at
 // once, which is what counts when a step has a handful of rows.  E a multiple of 4, E <= 256*VPL.
+// A workgroup is one wavefront (few rows: as many compute units as rows) or four (many rows: fewer,
+// fuller workgroups).
 template <int VPL>
-__global__ void __launch_bounds__(DA_WAVE)
+__global__ void __launch_bounds__(4 * DA_WAVE)
 layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
                      const void* __restrict__ w, int w_dtype, const void* __restrict__ b, int b_dtype,
-                     float eps, void* __restrict__ y, int y_dtype, int E) {
-  const int lane = threadIdx.x, r = blockIdx.x;
+                     float eps, void* __restrict__ y, int y_dtype, int R, int E) {
+  const int lane = threadIdx.x % DA_WAVE;
+  const int r = blockIdx.x * (blockDim.x / DA_WAVE) + threadIdx.x / DA_WAVE;
+  if (r >= R) return;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * E;
   float4 v[VPL];
   float s = 0.f;
@@ -168,10 +172,11 @@ extern "C" int da_layernorm(const float* x, const int* rows, const void* w, int 
   hipStream_t st = (hipStream_t)stream;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
                        (!b || (uintptr_t)b % 16 == 0);
+  const int wpb = R >= 512 ? 4 : 1;      // wavefronts (rows) per workgroup
   if (E % 4 == 0 && E <= 2048 && aligned) {
 #define LN_LAUNCH(V)                                                                                      \
-  hipLaunchKernelGGL(layernorm_row_kernel<V>, dim3(R), dim3(DA_WAVE), 0, st, x, rows, w, w_dtype, b, b_dtype, \
-                     eps, y, y_dtype, E)
+  hipLaunchKernelGGL(layernorm_row_kernel<V>, dim3(da_ceil_div(R, wpb)), dim3(wpb * DA_WAVE), 0, st, x, rows, w, \
+                     w_dtype, b, b_dtype, eps, y, y_dtype, R, E)
     if (E <= 256) LN_LAUNCH(1);
     else if (E <= 512) LN_LAUNCH(2);
     else if (E <= 1024) LN_LAUNCH(4);
@@ -211,6 +216,58 @@ __global__ void kv_write_kernel(const T* __restrict__ qkv, int ld, int k_off, in
   }
 }
 
+// The same for bfloat16 and many tokens: a workgroup takes 16 consecutive tokens.  Keys go over in
+// 16-byte pieces.  Where the 16 tokens fill 16 consecutive, aligned rows of one page (a prompt
+// portion that starts on such a boundary), a value column's 16 entries are one 32-byte run in the
+// dimension-major page and are stored as such; otherwise entry by entry.
+#define KVW_ROWS 16
+__global__ void __launch_bounds__(256)
+kv_write_rows_kernel(const bf16_t* __restrict__ qkv, int ld, int k_off, int v_off, bf16_t* __restrict__ cache,
+                     const int* __restrict__ slot_map, int N, int Hkv, int D, int page) {
+  __shared__ int slots[KVW_ROWS];
+  __shared__ int run;
+  const int n0 = blockIdx.x * KVW_ROWS;
+  if (threadIdx.x < KVW_ROWS) slots[threadIdx.x] = n0 + threadIdx.x < N ? slot_map[n0 + threadIdx.x] : -1;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int ok = slots[0] >= 0 && slots[0] % KVW_ROWS == 0;
+    for (int i = 1; i < KVW_ROWS; ++i) ok = ok && slots[i] == slots[0] + i;
+    run = ok;
+  }
+  __syncthreads();
+  const int W = Hkv * D, chunks = W / 8;
+  // blockIdx.y splits the columns, so that few tokens still fill the chip
+  const int t = threadIdx.x + blockIdx.y * blockDim.x, stride = blockDim.x * gridDim.y;
+  // keys: rows of 16-byte pieces
+  for (int e = t; e < KVW_ROWS * chunks; e += stride) {
+    const int i = e / chunks, c = (e % chunks) * 8, slot = slots[i];
+    if (slot < 0) continue;
+    const int h = c / D, d = c % D;
+    *(uint4*)(cache + cache_k_row(slot / page, h, slot % page, Hkv, page, D) + d) =
+        *(const uint4*)(qkv + (size_t)(n0 + i) * ld + k_off + c);
+  }
+  // values: a thread takes a column (head, dimension) of the 16 tokens
+  for (int c = t; c < W; c += stride) {
+    const int h = c / D, d = c % D;
+    bf16_t v[KVW_ROWS];
+#pragma unroll
+    for (int i = 0; i < KVW_ROWS; ++i) v[i] = slots[i] >= 0 ? qkv[(size_t)(n0 + i) * ld + v_off + c] : (bf16_t)0;
+    if (run) {
+      bf16_t* dst = cache + cache_v_base(slots[0] / page, h, Hkv, page, D) + (long long)d * page + slots[0] % page;
+      uint32_t u[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) u[i] = (uint32_t)v[2 * i] | ((uint32_t)v[2 * i + 1] << 16);
+      *(uint4*)dst = make_uint4(u[0], u[1], u[2], u[3]);
+      *(uint4*)(dst + 8) = make_uint4(u[4], u[5], u[6], u[7]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < KVW_ROWS; ++i)
+        if (slots[i] >= 0)
+          cache[cache_v_base(slots[i] / page, h, Hkv, page, D) + (long long)d * page + slots[i] % page] = v[i];
+    }
+  }
+}
+
 extern "C" int da_kv_write(const void* qkv, int dtype, int ld, int k_off, int v_off, void* cache,
                            const int* slot_map, int N, int Hkv, int D, int page, void* stream) {
   DA_REQUIRE(N >= 0 && Hkv > 0 && D > 0 && page > 0, "kv_write: bad sizes");
@@ -218,7 +275,12 @@ extern "C" int da_kv_write(const void* qkv, int dtype, int ld, int k_off, int v_
              "kv_write: k/v columns [%d,%d)+%d exceed the row length %d", k_off, v_off, Hkv * D, ld);
   if (N == 0) return 0;
   const int threads = 256;
-  if (dtype == DA_BF16)
+  const bool vec = dtype == DA_BF16 && N >= 256 && D % 8 == 0 && page % KVW_ROWS == 0 && ld % 8 == 0 &&
+                   k_off % 8 == 0 && ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)cache % 16 == 0);
+  if (vec)
+    hipLaunchKernelGGL(kv_write_rows_kernel, dim3(da_ceil_div(N, KVW_ROWS), da_ceil_div(Hkv * D, 256)), dim3(threads), 0, (hipStream_t)stream,
+                       (const bf16_t*)qkv, ld, k_off, v_off, (bf16_t*)cache, slot_map, N, Hkv, D, page);
+  else if (dtype == DA_BF16)
     hipLaunchKernelGGL(kv_write_kernel<bf16_t>, dim3(N), dim3(threads), 0, (hipStream_t)stream,
                        (const bf16_t*)qkv, ld, k_off, v_off, (bf16_t*)cache, slot_map, Hkv, D, page);
   else

@@ -353,6 +353,12 @@ def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+# Measured on MI355X (2,048 rows): in the tile kernel's epilogue the cache write doubles the product's
+# time (two-byte stores, scattered for the values); the write kernel after it costs half of that.  For a
+# handful of rows the epilogue saves a kernel.
+KV_EPILOGUE_MAX_ROWS = 64
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            act: Optional[str] = None, accumulate: bool = False, kv_cache: Optional[torch.Tensor] = None,
            slot_map: Optional[torch.Tensor] = None, q_cols: int = 0) -> torch.Tensor:
@@ -361,8 +367,11 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     ``kv_cache`` the k | v columns (from ``q_cols`` on) are also written to the cache rows
     ``slot_map``: in the product's epilogue on the matrix cores, by the write kernel otherwise."""
     if _MODE == "tuned" and _mfma_ok(a, w):
-        return linear_mfma(a, w, bias, out, act, accumulate, kv_cache, slot_map, q_cols)
-    linear_ref(a, w, bias, out, act, accumulate)
+        if kv_cache is None or a.shape[0] <= KV_EPILOGUE_MAX_ROWS:
+            return linear_mfma(a, w, bias, out, act, accumulate, kv_cache, slot_map, q_cols)
+        linear_mfma(a, w, bias, out, act, accumulate)
+    else:
+        linear_ref(a, w, bias, out, act, accumulate)
     if kv_cache is not None:
         _, _, Hkv, _, D = kv_cache.shape
         kv_write(out, q_cols, q_cols + Hkv * D, kv_cache, slot_map, Hkv, D)

@@ -266,6 +266,49 @@ def test_attention_reference_vector_shape(ops):
             assert np.abs(out2.double().cpu().numpy() - want).max() < tol
 
 
+@pytest.mark.parametrize("page", [16, 32, 64])
+@pytest.mark.parametrize("N", [40, 600])
+def test_cache_write_puts_every_key_and_value_in_its_row(ops, N, page):
+    """Both write kernels (a token a workgroup; 16 tokens a workgroup from 256 tokens on) against
+    direct placement: whole aligned pages in order, runs that start inside a page, single rows
+    all over, and tokens whose keys are not kept (-1)."""
+    Hq, Hkv, D = 3, 2, 48
+    g = torch.Generator().manual_seed(N + page)
+    n_pages = 4 * (N // page + 2)
+    free = torch.randperm(n_pages, generator=g).tolist()
+    slots = []
+    while len(slots) < N:
+        kind = len(slots) // 16 % 4
+        pg = free.pop()
+        if kind == 0:      # a whole page in order
+            slots += [pg * page + i for i in range(page)]
+        elif kind == 1:    # a run that starts inside the page
+            slots += [pg * page + i for i in range(5, page)]
+        elif kind == 2:    # rows of a page in any order
+            slots += [pg * page + int(i) for i in torch.randperm(page, generator=g)[:11]]
+        else:              # not kept
+            slots += [-1] * 7
+    slots = slots[:N]
+    qkv = bf(torch.randn(N, (Hq + 2 * Hkv) * D, generator=g)).to(DEV)
+    st = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    for dtype in (torch.bfloat16, torch.float32):
+        x = qkv.to(dtype)
+        cache = torch.zeros(n_pages, 2, Hkv, page, D, dtype=dtype, device=DEV)
+        ops.kv_write(x, Hq * D, (Hq + Hkv) * D, cache, st, Hkv, D)
+        want = torch.zeros(n_pages, 2, Hkv, page, D, dtype=dtype)
+        want_v = torch.zeros(n_pages, Hkv, D, page, dtype=dtype)          # values lie dimension-major in a page
+        xc = x.cpu()
+        for n, sl in enumerate(slots):
+            if sl < 0:
+                continue
+            pg, row = divmod(sl, page)
+            want[pg, 0, :, row, :] = xc[n, Hq * D:(Hq + Hkv) * D].view(Hkv, D)
+            want_v[pg, :, :, row] = xc[n, (Hq + Hkv) * D:].view(Hkv, D)
+        got = cache.cpu()
+        assert torch.equal(got[:, 0], want[:, 0])
+        assert torch.equal(got[:, 1].reshape(n_pages, Hkv, D, page), want_v)
+
+
 def test_a_far_key_among_hundreds_is_found(ops):
     """Random keys give near-uniform weights, which would hide a lost key: here one key far back
     carries almost all the weight of the last query."""

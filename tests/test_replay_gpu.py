@@ -105,6 +105,45 @@ def test_long_decoding_and_first_tokens(model_a, dtype):
     helpers.check_against_plain(m, got, [("f", ids[:5])], dtype, "first tokens")
 
 
+BENCH_SIZES = {   # the layer sizes of the models that the benchmark runs, two layers of each
+    "124m": dict(n_embd=768, n_head=12),
+    "1.5b": dict(n_embd=1600, n_head=25),
+}
+
+
+@pytest.mark.parametrize("size", sorted(BENCH_SIZES))
+def test_layer_sizes_of_the_benchmark_models(size, tmp_path_factory):
+    """GPT-2 124M and 1.5B layer sizes (width, heads of 64, 4x inner width, the vocabulary of 50,257
+    that is no multiple of anything, 1,024 positions), two layers, against the plain model: one
+    request of 200 tokens (several key tiles, pages in any order) cut into portions and single
+    tokens beside a second request, in 32-bit and in bfloat16.
+
+    Logits here are four times those of the tiny models (rms 0.55 to 0.8 against 0.16 to 0.2), and
+    bfloat16 errors grow with them, so the bfloat16 bound is taken relative to the logits' rms: the
+    largest error below 4 % of it and the rms error below 2^-7 of it (four bfloat16 roundings).  On
+    the tiny models the absolute bound of the other tests is 7 to 9 % of the rms.  The 32-bit bound
+    is the absolute one of the other tests."""
+    cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, vocab_size=50257, n_positions=1024,
+               layer_norm_epsilon=1e-5, activation_function="gelu_new", bos_token_id=50256, eos_token_id=50256,
+               **BENCH_SIZES[size])
+    m = helpers.make_model(tmp_path_factory.mktemp("bench_" + size.replace(".", "_")), cfg, seed=5)
+    reqs = [("long", m.prompt(200)), ("short", m.prompt(75, salt=1))]
+    steps = helpers.trace_mixed(reqs, seed=3, max_live=2, prefill_sizes=(130, 2, 37, 64), decode_tail=6)
+    for dtype in DTYPES:
+        s = session_for(m, dtype, helpers.max_live_tokens(steps))
+        got = helpers.replay(s, steps)
+        if dtype == "float32":
+            helpers.check_against_plain(m, got, reqs, dtype, f"{size} sizes")
+        else:
+            for rid, ids in reqs:
+                ref = m.plain_logits(ids)
+                err = np.abs(got[rid].astype(np.float64) - ref)
+                rms = np.sqrt((ref ** 2).mean())
+                assert err.max() <= 4e-2 * rms, (rid, err.max(), rms, int(np.argmax(err.max(axis=1))))
+                assert np.sqrt((err ** 2).mean()) <= 2.0 ** -7 * rms
+        s.cache.manager.check()
+
+
 @pytest.mark.parametrize("page_size", [16, 32, 64])
 def test_page_sizes(model_b, page_size):
     m = model_b
