@@ -1,7 +1,7 @@
 // Paged attention for decode rows in bfloat16: one query row per sequence.
 //
-// One workgroup of 16 wavefronts per (sequence, query head).  The keys lo..p of the sequence
-// are walked in aligned chunks of 64; wavefront v takes chunks v, v+16, ... (one each up to a
+// One workgroup of 8 wavefronts per (sequence, query head).  The keys lo..p of the sequence
+// are walked in aligned chunks of 64; wavefront v takes chunks v, v+8, ... (two each at a
 // context of 1,024).  All loads of a phase are issued before any is used, so a chunk costs two
 // memory round trips.
 //   scores : CPR lanes share a key, each holding a 16-byte piece of the key row and the matching
@@ -17,7 +17,6 @@
 // Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:504-532;
 // tensor/src/main/java/io/teknek/deliverance/tensor/operations/TensorOperations.java:240-272.
 #include "common.h"
-#include <stdlib.h>
 
 #define DEC_MAX_D 256
 #define DEC_DPL (DEC_MAX_D / DA_WAVE)   // value dimensions per lane at most
@@ -197,20 +196,14 @@ extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const 
              "attn_decode: q and the cache must be 16-byte aligned");
   if (S == 0) return 0;
   const int pieces = D / 8;
-  static int waves = -1;
-  if (waves < 0) { const char* e = getenv("DA_DECODE_WAVES"); waves = e ? atoi(e) : 8; }
+  // 8 wavefronts: 16 cost more to start than they hide, 4 leave a context of 1,024 two chunks deep
   dim3 grid(S * Hq);
   hipStream_t st = (hipStream_t)stream;
 #define LAUNCH2(C, W)                                                                                      \
   hipLaunchKernelGGL((attn_decode_kernel<C, W>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld,   \
                      (const bf16_t*)cache, block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, \
                      (bf16_t*)out, out_ld)
-#define LAUNCH(C)                                                  \
-  do {                                                             \
-    if (waves == 16) LAUNCH2(C, 16);                               \
-    else if (waves == 4) LAUNCH2(C, 4);                            \
-    else LAUNCH2(C, 8);                                            \
-  } while (0)
+#define LAUNCH(C) LAUNCH2(C, 8)
   if (pieces <= 2) LAUNCH(2);
   else if (pieces <= 4) LAUNCH(4);
   else if (pieces <= 8) LAUNCH(8);

@@ -8,7 +8,8 @@
 //  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
 //    buffers, with the next four slabs already in flight in registers.  For steps with many rows
 //    (prefill).
-//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows; its
+//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows (or, with few
+//    columns, some of the 16-row tiles); its
 //    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
 //    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
 //
@@ -253,6 +254,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   __shared__ float red[NW][MT * 16][SK_COLS + 1];
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int n0 = blockIdx.x * SK_COLS;
+  const int r0 = blockIdx.y * MT * 16;             // the workgroup's first row
   const int fr = lane % 16, fk = (lane / 16) * 8;
   floatx4 acc[MT];
 #pragma unroll
@@ -264,8 +266,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   const bf16_t* ap[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
-    arow_ok[i] = i * 16 + fr < M;
-    ap[i] = a + (size_t)(arow_ok[i] ? i * 16 + fr : 0) * lda + fk;
+    arow_ok[i] = r0 + i * 16 + fr < M;
+    ap[i] = a + (size_t)(arow_ok[i] ? r0 + i * 16 + fr : 0) * lda + fk;
   }
   // what the epilogue needs is asked for first, so that it has arrived when the products are done
   constexpr int EPT = (MT * 16 * SK_COLS + NW * 64 - 1) / (NW * 64);     // output elements per thread
@@ -273,7 +275,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   int e_slot[EPT];
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, m = e / SK_COLS, n = n0 + e % SK_COLS;
+    const int e = t + j * NW * 64, m = r0 + e / SK_COLS, n = n0 + e % SK_COLS;
     const bool ok = e < MT * 16 * SK_COLS && m < M && n < N;
     e_bias[j] = (ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
     e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
@@ -308,11 +310,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, m = e / SK_COLS, c = e % SK_COLS, n = n0 + c;
+    const int e = t + j * NW * 64, ml = e / SK_COLS, m = r0 + ml, c = e % SK_COLS, n = n0 + c;
     if (e < MT * 16 * SK_COLS && m < M && n < N) {
-      float v = red[0][m][c];
+      float v = red[0][ml][c];
 #pragma unroll
-      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][m][c];
+      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][ml][c];
       v = apply_act(v + e_bias[j], ep.act);
       const size_t o = (size_t)m * ep.ldo + n;
       if (ep.accumulate) ((float*)ep.out)[o] = e_old[j] + v;
@@ -326,6 +328,14 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 template <int NW>
 static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
                           const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
+  // With few columns the row tiles are spread over more workgroups (blockIdx.y), as long as the chip
+  // is not full: each then reads fewer rows of a.  A row's sums do not depend on it.
+  for (int mb = 1; mb < mt; mb *= 2)
+    if ((long)grid.x * da_ceil_div(mt, mb) <= 256) {
+      grid.y = da_ceil_div(mt, mb);
+      mt = mb;
+      break;
+    }
   // few rows leave registers for more chunks in flight
   if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
   else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
