@@ -44,7 +44,8 @@ __device__ __forceinline__ void load8_param(const void* p, int dtype, int i, flo
 }
 
 template <int MT, int NW, int FZ_UNROLL>
-__global__ void __launch_bounds__(NW * 64)
+// (for one row tile the registers are held to 128, so that two workgroups of 8 wavefronts share a compute unit)
+__global__ void __launch_bounds__(NW * 64, MT == 1 ? 4 : 1)
 gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
                       int M, int N, int K) {
   __shared__ float red[NW][MT * 16][FZ_COLS + 1];
@@ -66,8 +67,7 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
       const int k = k0 + u * NW * 32;
       const bool kin = k + fk < K;
       const int ks = kin ? k : -fk;
-      wv[u] = load16(wp + ks);
-      if (!(kin && wrow_ok)) wv[u] = zero;
+      wv[u] = load16(wp + ks);      // past K: the row's first chunk, met by zeros in a; past N: row 0, never stored
       load8_param(ln.g, ln.g_dtype, ks + fk, gg[u]);
       if (ln.b) load8_param(ln.b, ln.b_dtype, ks + fk, bb[u]);
     }
@@ -93,9 +93,8 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 #pragma unroll
     for (int i = 0; i < FZ_VPL; ++i) {
       const int c = (lane + i * 64) * 4;
-      v[i] = *(const float4*)(xr + (c < K ? c : 0));          // never a conditional load
-      if (c >= K) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+      v[i] = *(const float4*)(xr + (c < K ? c : 0));          // never a conditional load, nor a value replaced
+      s += (c < K ? 1.f : 0.f) * ((v[i].x + v[i].y) + (v[i].z + v[i].w));
     }
     const float mean = wave_sum(s) / (float)K;
     float q = 0.f;

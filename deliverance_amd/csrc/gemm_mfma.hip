@@ -21,6 +21,7 @@
 // row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
 // l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
 #include "gemm_common.h"
+#include <type_traits>
 
 #define BKT 64               // k per slab
 #define LDS_LD (BKT + 8)     // padded row length in elements (144 bytes): spreads rows over banks
@@ -259,7 +260,6 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   floatx4 acc[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const uint4 zero = make_uint4(0, 0, 0, 0);
   const bool wrow_ok = n0 + fr < N;
   const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
   bool arow_ok[MT];
@@ -281,27 +281,47 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
     e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
     e_slot[j] = (ok && kv.cache) ? kv.slot_map[m] : -1;
   }
-  for (int k0 = wave * 32; k0 < K; k0 += NW * 32 * SK_UNROLL) {
-    uint4 wv[SK_UNROLL], av[SK_UNROLL][MT];
+  // The wavefront's whole chunks go in groups of SK_UNROLL, then of half that, and so on down to
+  // one: a group is nothing but its loads, all in flight at once, and then its products.  (A value
+  // replaced after its load, like a zero past K, makes the compiler wait for that load and all
+  // before it; that is left to the one chunk that K may cut.)  Rows past M and columns past N read
+  // row 0: what they give is never stored.
+  int k0 = wave * 32;
+  int left = k0 + 32 <= K ? (K - 32 - k0) / (NW * 32) + 1 : 0;        // whole chunks of this wavefront
+  auto group = [&](auto gc) {
+    constexpr int G = decltype(gc)::value;
+    uint4 wv[G], av[G][MT];
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
-      const int k = k0 + u * NW * 32;
-      const bool kin = k + fk < K;
-      const int ks = kin ? k : -fk;             // a load that is not wanted reads the row's first chunk and is dropped
-      wv[u] = load16(wp + ks);
-      if (!(kin && wrow_ok)) wv[u] = zero;
+    for (int u = 0; u < G; ++u) {
+      wv[u] = load16(wp + k0 + u * NW * 32);
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        av[u][i] = load16(ap[i] + ks);
-        if (!(kin && arow_ok[i])) av[u][i] = zero;
-      }
+      for (int i = 0; i < MT; ++i) av[u][i] = load16(ap[i] + k0 + u * NW * 32);
     }
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u)
+    for (int u = 0; u < G; ++u)
 #pragma unroll
       for (int i = 0; i < MT; ++i)
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u][i]),
                                                          __builtin_bit_cast(bf16x8_t, wv[u]), acc[i], 0, 0, 0);
+    k0 += G * NW * 32;
+    left -= G;
+  };
+  while (left >= SK_UNROLL) group(std::integral_constant<int, SK_UNROLL>{});
+  if (SK_UNROLL > 4 && left >= 4) group(std::integral_constant<int, 4>{});
+  if (SK_UNROLL > 2 && left >= 2) group(std::integral_constant<int, 2>{});
+  if (left >= 1) group(std::integral_constant<int, 1>{});
+  if (k0 < K) {                                 // the chunk that K cuts (K is a multiple of 8, a chunk is 32 wide)
+    const bool kin = k0 + fk < K;
+    const int ks = kin ? k0 : -fk;              // a load that is not wanted reads the row's first chunk and is dropped
+    uint4 wv = load16(wp + ks);
+    if (!kin) wv = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      uint4 av = load16(ap[i] + ks);
+      if (!kin) av = make_uint4(0, 0, 0, 0);
+      acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                       __builtin_bit_cast(bf16x8_t, wv), acc[i], 0, 0, 0);
+    }
   }
 #pragma unroll
   for (int i = 0; i < MT; ++i)

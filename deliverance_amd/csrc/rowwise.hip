@@ -120,15 +120,20 @@ layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
   const int r = blockIdx.x * (blockDim.x / DA_WAVE) + threadIdx.x / DA_WAVE;
   if (r >= R) return;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * E;
-  float4 v[VPL];
+  // every load of the row, of the gain and of the bias is asked for at once (past the row's end
+  // the row's start is read and left out of the sums), before anything is reduced
+  float4 v[VPL], g[VPL], bb[VPL];
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
-    v[i] = *(const float4*)(xr + (c < E ? c : 0));          // never a conditional load
-    if (c >= E) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    v[i] = *(const float4*)(xr + (c < E ? c : 0));
+    g[i] = load_param4(w, w_dtype, c < E ? c : 0);
+    bb[i] = b ? load_param4(b, b_dtype, c < E ? c : 0) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
+#pragma unroll
+  for (int i = 0; i < VPL; ++i)
+    s += ((lane + i * DA_WAVE) * 4 < E ? 1.f : 0.f) * ((v[i].x + v[i].y) + (v[i].z + v[i].w));
   const float mean = wave_sum(s) / (float)E;
   float q = 0.f;
 #pragma unroll
@@ -144,13 +149,8 @@ layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
     if (c < E) {
-      const float4 g = load_param4(w, w_dtype, c);
-      float4 o = make_float4((v[i].x - mean) * inv * g.x, (v[i].y - mean) * inv * g.y,
-                             (v[i].z - mean) * inv * g.z, (v[i].w - mean) * inv * g.w);
-      if (b) {
-        const float4 bb = load_param4(b, b_dtype, c);
-        o.x += bb.x; o.y += bb.y; o.z += bb.z; o.w += bb.w;
-      }
+      const float4 o = make_float4((v[i].x - mean) * inv * g[i].x + bb[i].x, (v[i].y - mean) * inv * g[i].y + bb[i].y,
+                                   (v[i].z - mean) * inv * g[i].z + bb[i].z, (v[i].w - mean) * inv * g[i].w + bb[i].w);
       if (y_dtype == DA_BF16) {
         uint2 u;
         u.x = (uint32_t)f32_to_bf16(o.x) | ((uint32_t)f32_to_bf16(o.y) << 16);

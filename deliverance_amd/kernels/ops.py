@@ -302,8 +302,9 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     return out
 
 
-# Measured on MI355X: the fused kernel wins up to 8 rows and a width of 1024; beyond, the separate
-# norm and product are faster (every 16 output columns recompute the rows' statistics).
+# Measured on MI355X inside the model: the fused kernel wins up to 8 rows and a width of 1024 (by
+# 2 to 3 % of a decode step); beyond, the separate norm and product are faster (every 16 output
+# columns recompute the rows' statistics, and a wavefront's loads come in more rounds).
 FUSED_LN_MAX_ROWS = 8
 FUSED_LN_MAX_K = 1024
 FUSED_LN_MAX_N = 16384      # ... and never for a vocabulary
