@@ -57,6 +57,44 @@ def step_flops(c, seq_lens_new, past=0):
     return gemm + attn
 
 
+def mixed_run(args, cfg, folder, rng, dkey):
+    """Continuous batching under load: every request arrives at once; the scheduler admits them as
+    seats and pages allow, cuts prompts into portions of at most 512 tokens and runs them in the
+    same steps as the other requests' decoding.  One JSON line: generated tokens a second over the
+    whole run (prompt processing included)."""
+    import torch
+    from deliverance_amd import AutoModelForCausalLM, GeneratorParameters
+    n_req, new = 64, 128
+    longest = cfg["n_positions"] - new - 1
+    model = AutoModelForCausalLM.from_pretrained(
+        folder, dtype=args.dtype, max_num_seqs=n_req, max_batch_tokens=512 + n_req, max_chunk=512,
+        max_cached_tokens=n_req * cfg["n_positions"], page_size=16)
+    lengths = [int(x) for x in rng.integers(16, longest + 1, size=n_req)]
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)] for n in lengths]
+    params = GeneratorParameters(max_tokens=new, ignore_eos=True)
+    best = None
+    for _ in range(2):                        # the first run records the decode graphs
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = model.generate(prompts, params)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    assert all(len(o.generated_tokens) == new for o in outs)
+    stats = model.stats()
+    print(json.dumps({
+        "metric": "generated tok/s, %d requests at once (GPT-2 %s layer sizes, prompts 16..%d, %d new tokens each, "
+                  "prompt portions of 512 beside decoding)" % (n_req, args.model, longest, new),
+        "value": round(n_req * new / best, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+        "dtype": dkey, "data": "synthetic (random weights, uniform-random token ids)",
+        "seconds": round(best, 4), "prompt_tokens": sum(lengths), "generated_tokens": n_req * new,
+        "all_tokens_per_second": round((sum(lengths) + n_req * new) / best, 1),
+        "config": {"model": "gpt2-" + args.model, "n_layer": cfg["n_layer"], "n_embd": cfg["n_embd"],
+                   "n_head": cfg["n_head"], "requests": n_req, "max_chunk": 512, "page_size": 16,
+                   "preemptions": stats.get("preemptions", 0)}}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,6 +107,9 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+                    help="mixed: 64 requests with prompts of 16 to 895 tokens arrive at once, prompt portions of 512 "
+                         "tokens run beside the decoding of the others, 128 new tokens each (use --model 355m)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -121,6 +162,8 @@ def main():
             model.scheduler.finished.clear()
             return dt, ctx_mean
 
+        if args.workload == "mixed":
+            return mixed_run(args, cfg, folder, rng, dkey)
         model = engine(max(args.batch, 64 if not args.no_points else args.batch))
         dt, ctx_mean = decode_run(model, args.batch, args.steps, args.warmup)
         ms_per_step = dt / args.steps * 1e3

@@ -109,11 +109,11 @@ class CausalLanguageModel:
         """One scheduler decision and one model step with its sampling.  Returns the requests
         whose end became known in this call.
 
-        A step whose tokens are all sampled on the device may be left running when the call
-        returns.  The next call then first launches the step after it (taking its tokens from the
-        device, ``Scheduler.schedule_ahead``) and only then reads the older step's tokens, so
-        the host's work for one step runs beside the device's work for the step before.  When
-        the next step cannot be decided ahead, the older step is read first, as without this."""
+        A step may be left running when the call returns.  The next call then first launches the
+        step after it (``Scheduler.schedule_ahead``; tokens that are still being sampled are taken
+        on the device) and only then reads the older step's tokens, so the host's work for one
+        step runs beside the device's work for the step before.  When the next step cannot be
+        decided ahead (pages are short), the older step is read first, as without this."""
         done: List[Request] = []
         if self._inflight is not None:
             ahead = self._launch_ahead(self._inflight)
@@ -142,8 +142,7 @@ class CausalLanguageModel:
         return self._retire(flight)
 
     def _may_stay_in_flight(self, flight: "_InFlight") -> bool:
-        return (self.engine_config.run_ahead and bool(flight.samplers) and flight.lp is None
-                and len(flight.samplers) == len(flight.batch))
+        return self.engine_config.run_ahead and flight.lp is None
 
     def _launch_ahead(self, prev: "_InFlight") -> Optional["_InFlight"]:
         if any(s.request.params.log_probs and s.request.params.top_log_probs > 0 for s in prev.batch):
@@ -157,17 +156,19 @@ class CausalLanguageModel:
 
     def _launch(self, batch: List[Scheduled], sampled_row: Optional[Dict[int, int]]) -> "_InFlight":
         """Put one step on the device: model, sampling, and the copy of the sampled tokens to the
-        host.  With ``sampled_row`` every entry's token is the one the step before sampled for the
-        same request (row ``sampled_row[id(request)]`` of the runner's sampled tokens)."""
+        host.  An entry whose token the host does not know yet takes the one the step before
+        sampled for the same request (row ``sampled_row[id(request)]`` of the runner's sampled
+        tokens)."""
         V = self.config.vocab_size
         entries = []
         records: List[int] = []
         samplers: List[Scheduled] = []
         for s in batch:
             req = s.request
-            if sampled_row is None:
+            if s.start + s.n <= req.n_tokens:
                 entries.append(StepEntry(req.rid, req.tokens_from(s.start, s.n), [s.n - 1] if s.samples else []))
-            else:
+            else:       # the one token that the running step is still sampling
+                assert sampled_row is not None and s.n == 1 and s.start == req.n_tokens
                 entries.append(StepEntry(req.rid, [0], [0], from_sampled=sampled_row[id(req)]))
             if s.samples:
                 records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))

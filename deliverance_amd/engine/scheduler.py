@@ -18,9 +18,11 @@ this engine's own:
   again from its tokens (prompt and what it has generated).  A request that is alone and still
   cannot fit fails with ``finish_reason = "error"``.
 * ``schedule_ahead`` decides the step after one that is still running, before its tokens are
-  known, when that decision cannot depend on them: every running request gets its next decode
-  step, except those that end by length.  A request that turns out to have sampled an end token
-  has then one step too many in flight; its result is dropped when that step is booked.
+  known: requests that sampled there decode the token that is still on the device (those that end
+  by length leave), prompts get their next portions, waiting requests are admitted.  Only when
+  pages run short does it decline: preemption is decided with the tokens known.  A request that
+  turns out to have sampled an end token has then one step too many in flight; its result is
+  dropped when that step is booked.
 """
 from __future__ import annotations
 
@@ -121,7 +123,7 @@ class Scheduler:
         ps = self.cache.page_size
         if opened:
             have = len(self.cache.table(req.rid, 0)) * ps if self.cache.groups else 10 ** 9
-            base = self.cache.length(req.rid)
+            base = self.cache.length(req.rid) + self.cache.pending(req.rid)
         else:
             have, base = 0, 0
         free = min((p.n_free for p in self.cache.pools), default=10 ** 9)
@@ -146,6 +148,29 @@ class Scheduler:
         req.t_finish = time.perf_counter()
         self.finished.append(req)
         self.counters["finished"] += 1
+
+    def _admit(self, batch: List[Scheduled], budget: int) -> None:
+        """Admission, in arrival order, never at a running request's cost."""
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and self.cache.can_open():
+            req = self.waiting[0]
+            want = min(req.n_tokens, budget, self.max_chunk)
+            n = self._fit(req, want, False)
+            if n == 0:
+                if not self.running and not batch:
+                    self.waiting.popleft()
+                    self._fail(req, "the cache pool cannot hold a single page for the request")
+                    continue
+                break
+            self.waiting.popleft()
+            slot = self.cache.open(req.rid)
+            if self.on_open is not None:
+                self.on_open(slot)
+            req.state = RUNNING
+            self.running.append(req)
+            self.counters["admitted"] += 1
+            start = self.cache.extend(req.rid, n)
+            batch.append(Scheduled(req, start, n, start + n == req.n_tokens))
+            budget -= n
 
     def schedule(self) -> List[Scheduled]:
         """Pick this step's work and reserve its cache positions."""
@@ -181,27 +206,7 @@ class Scheduler:
                 start = self.cache.extend(req.rid, n)
                 batch.append(Scheduled(req, start, n, start + n == req.n_tokens))
                 budget -= n
-        # admission, in arrival order, never at a running request's cost
-        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and self.cache.can_open():
-            req = self.waiting[0]
-            want = min(req.n_tokens, budget, self.max_chunk)
-            n = self._fit(req, want, False)
-            if n == 0:
-                if not self.running and not batch:
-                    self.waiting.popleft()
-                    self._fail(req, "the cache pool cannot hold a single page for the request")
-                    continue
-                break
-            self.waiting.popleft()
-            slot = self.cache.open(req.rid)
-            if self.on_open is not None:
-                self.on_open(slot)
-            req.state = RUNNING
-            self.running.append(req)
-            self.counters["admitted"] += 1
-            start = self.cache.extend(req.rid, n)
-            batch.append(Scheduled(req, start, n, start + n == req.n_tokens))
-            budget -= n
+        self._admit(batch, budget)
         if batch:
             self.counters["steps"] += 1
             self.counters["batch_tokens"] += sum(s.n for s in batch)
@@ -215,31 +220,50 @@ class Scheduler:
                 or req.n_tokens + more > req.limit)
 
     def schedule_ahead(self, inflight: List[Scheduled]) -> Optional[List[Scheduled]]:
-        """The batch that follows ``inflight`` (scheduled, launched, not yet completed), or None
-        when it can only be decided after ``complete``: someone waits and could be admitted, a
-        running request is not at its last token in ``inflight``, or pages are short (preemption
-        needs the tokens).  Nothing is reserved when None is returned."""
-        if self.waiting and len(self.running) < self.max_num_seqs and self.cache.can_open():
-            return None
+        """The batch that follows ``inflight`` (scheduled, launched, not yet completed), decided
+        without its tokens: a request that sampled in ``inflight`` decodes the token that is still on
+        the device (unless it ends by length), a request in its prompt gets its next portion, waiting
+        requests are admitted as in ``schedule``.  Returns None, with nothing reserved, when a running
+        request cannot get all the pages it asks for: who gives way then is decided with the tokens
+        known."""
         last = {id(s.request): s for s in inflight}
-        nxt: List[Request] = []
-        for req in self.running:
-            s = last.get(id(req))
-            if s is None or not s.samples or s.start + s.n != req.n_tokens:
-                return None
-            if not self._ends_by_length(req, 1):
-                nxt.append(req)
-        if not nxt or len(nxt) > self.max_batch_tokens:
+        G = len(self.cache.pools)
+        need = [0] * G
+        free = [p.n_free for p in self.cache.pools]
+        budget = self.max_batch_tokens
+        plan = []
+        for phase in (1, 0):
+            for req in self.running:
+                s = last.get(id(req))
+                if s is None:
+                    done, total = req.n_computed, req.n_tokens
+                else:
+                    if s.samples and self._ends_by_length(req, 1):
+                        continue                    # ends when ``inflight`` is completed
+                    done, total = s.start + s.n, req.n_tokens + (1 if s.samples else 0)
+                left = total - done
+                if left <= 0:
+                    return None
+                if (left == 1) != bool(phase) or budget <= 0:
+                    continue
+                want = min(left, budget, self.max_chunk)
+                pages = self.cache.pages_needed(req.rid, want)
+                if any(need[g] + pages[g] > free[g] for g in range(G)):
+                    return None
+                for g in range(G):
+                    need[g] += pages[g]
+                plan.append((req, done, want, done + want == total))
+                budget -= want
+        batch = []
+        for req, start, n, samples in plan:
+            got = self.cache.extend(req.rid, n)
+            assert got == start, "reserved positions follow the running step's"
+            batch.append(Scheduled(req, start, n, samples))
+        self._admit(batch, budget)
+        if not batch:
             return None
-        need = [0] * len(self.cache.pools)
-        for req in nxt:
-            for g, n in enumerate(self.cache.pages_needed(req.rid, 1)):
-                need[g] += n
-        if any(n > pool.n_free for n, pool in zip(need, self.cache.pools)):
-            return None
-        batch = [Scheduled(req, self.cache.extend(req.rid, 1), 1, True) for req in nxt]
         self.counters["steps"] += 1
-        self.counters["batch_tokens"] += len(batch)
+        self.counters["batch_tokens"] += sum(s.n for s in batch)
         return batch
 
     # ---- after the step ----------------------------------------------------------------------

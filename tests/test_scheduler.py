@@ -191,10 +191,16 @@ def drive_ahead(s, cache, max_steps=10000):
     steps were decided ahead."""
     inflight = None          # (batch, sampled tokens by request id), launched but not completed
     n_ahead = 0
+    reached = {}             # request -> (positions launched so far, preemptions seen): no gap, no repeat
 
     def launch(batch, prev):
         sampled = {}
         for b in batch:
+            at, pre = reached.get(b.request.rid, (0, b.request.n_preempted))
+            if pre != b.request.n_preempted:
+                at = 0                                         # preempted: computed again from the start
+            assert b.start == at, f"{b.request.rid}: portion starts at {b.start}, {at} positions were launched"
+            reached[b.request.rid] = (b.start + b.n, b.request.n_preempted)
             if b.samples:
                 toks = b.request.tokens_from(0, min(b.start + b.n, b.request.n_tokens))
                 if b.start + b.n > b.request.n_tokens:         # its last token is the one the older step sampled
@@ -209,7 +215,12 @@ def drive_ahead(s, cache, max_steps=10000):
             launched = None
             if nxt is not None:
                 n_ahead += 1
-                assert all(b.n == 1 and b.samples and b.start == b.request.n_tokens for b in nxt)
+                for b in nxt:        # only the token that is still being sampled may be unknown
+                    if b.start + b.n > b.request.n_tokens:
+                        assert b.n == 1 and b.samples and b.start == b.request.n_tokens
+                        assert b.request.rid in inflight[1]
+                assert sum(b.n for b in nxt) <= s.max_batch_tokens and all(b.n <= s.max_chunk for b in nxt)
+                assert len({id(b.request) for b in nxt}) == len(nxt)
                 launched = launch(nxt, inflight[1])
             s.complete(inflight[0], {rid: t for rid, t in inflight[1].items()})
             cache.check()
@@ -243,32 +254,42 @@ def test_steps_decided_ahead_give_the_same_tokens():
     assert cache.pools[0].n_free == cache.pools[0].n_pages and cache.live() == []
 
 
-def test_a_step_is_not_decided_ahead_when_it_could_depend_on_the_tokens():
+def test_what_is_decided_ahead_and_what_waits_for_the_tokens():
     s, cache = make(n_pages=3, page=4, max_num_seqs=2)
     a = s.add("a", [1, 2, 3], GeneratorParameters(max_tokens=20, ignore_eos=True))
     batch = s.schedule()
-    # someone waits and a seat is free: admission comes first
+    assert [(x.request.rid, x.start, x.n, x.samples) for x in batch] == [("a", 0, 3, True)]
+    # b arrives while a's prompt runs: a decodes the token that is still being sampled, b is admitted
     b = s.add("b", [4, 5], GeneratorParameters(max_tokens=20, ignore_eos=True))
-    assert s.schedule_ahead(batch) is None
+    ahead = s.schedule_ahead(batch)
+    assert [(x.request.rid, x.start, x.n, x.samples) for x in ahead] == [("a", 3, 1, True), ("b", 0, 2, True)]
+    assert cache.length("a") == 0 and cache.pending("a") == 4        # both steps' positions are reserved
     s.complete(batch, {"a": 5})
-    batch = s.schedule()                       # a decodes, b starts
-    assert {x.request.rid for x in batch} == {"a", "b"}
-    ahead = s.schedule_ahead(batch)            # both at their last token: decided ahead, positions reserved on top
-    assert ahead is not None and [x.start for x in ahead] == [4, 2]
+    assert cache.length("a") == 3 and cache.pending("a") == 1
+    batch, ahead = ahead, s.schedule_ahead(ahead)
+    assert [(x.request.rid, x.start, x.n) for x in ahead] == [("a", 4, 1), ("b", 2, 1)]
+    assert cache.pools[0].n_free == 0                                # a holds 2 pages (5 positions), b 1 (3 positions)
     s.complete(batch, {"a": 6, "b": 7})
-    s.complete(ahead, {"a": 8, "b": 9})
-    cache.check()
-    # a holds 2 pages (5 positions), b 1 (3 positions): the pool of 3 is spent
-    batch = s.schedule()                       # a at position 5, b at 3: both still fit their pages
-    assert [x.start for x in batch] == [5, 3] and cache.pools[0].n_free == 0
+    batch, ahead = ahead, s.schedule_ahead(ahead)                    # a at 5, b at 3: both still fit their pages
+    assert [(x.request.rid, x.start, x.n) for x in ahead] == [("a", 5, 1), ("b", 3, 1)]
+    s.complete(batch, {"a": 8, "b": 9})
     # b's position 4 needs a page that is not there: who gives way is decided with the tokens known
-    assert s.schedule_ahead(batch) is None
-    assert cache.length("a") == 5 and cache.length("b") == 3
+    assert s.schedule_ahead(ahead) is None
+    assert cache.length("a") == 5 and cache.pending("a") == 1 and cache.length("b") == 3 and cache.pending("b") == 1
     cache.check()
-    s.complete(batch, {"a": 10, "b": 11})
+    s.complete(ahead, {"a": 10, "b": 11})
     batch = s.schedule()
     # b gave its page back and starts again from its tokens, as far as the one free page reaches
     assert [(x.request.rid, x.start, x.n) for x in batch] == [("a", 6, 1), ("b", 0, 4)] and b.n_preempted == 1
+    # a prompt in portions goes on ahead as well: nothing of it depends on a token
+    s2, cache2 = make(max_chunk=4, max_batch_tokens=6)
+    c = s2.add("c", list(range(10)), GeneratorParameters(max_tokens=3, ignore_eos=True))
+    first = s2.schedule()
+    second = s2.schedule_ahead(first)
+    third = s2.schedule_ahead(second)
+    fourth = s2.schedule_ahead(third)
+    assert [[(x.start, x.n, x.samples) for x in st] for st in (first, second, third, fourth)] == \
+        [[(0, 4, False)], [(4, 4, False)], [(8, 2, True)], [(10, 1, True)]]
 
 
 @pytest.mark.parametrize("seed", range(4))
