@@ -19,7 +19,6 @@
 #include "common.h"
 
 #define DEC_MAX_D 256
-#define DEC_DPL (DEC_MAX_D / DA_WAVE)   // value dimensions per lane at most
 
 // CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
 template <int CPR, int DEC_WAVES>
@@ -29,8 +28,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
                    const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
                    int window, bf16_t* __restrict__ out, int out_ld) {
   constexpr int G = DA_WAVE / CPR;            // keys scored side by side
+  constexpr int DPL = CPR <= 8 ? 1 : CPR / 8; // value dimensions per lane: D <= 8 * CPR <= 64 * DPL
   __shared__ __attribute__((aligned(16))) float ps[DEC_WAVES][DA_WAVE];
-  __shared__ float part_acc[DEC_WAVES][DEC_MAX_D];
+  __shared__ float part_acc[DEC_WAVES][DPL * DA_WAVE];
   __shared__ float part_m[DEC_WAVES], part_l[DEC_WAVES];
 
   const int s = blockIdx.x / Hq, h = blockIdx.x % Hq;
@@ -39,6 +39,11 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   const int p = seq_lens[s] - 1;                      // the row's position; it sees keys lo..p
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int* bt = block_table + (size_t)s * max_blocks;
+  // addressing by shifts: the page size is a power of two (checked on the host)
+  const int lg = 31 - __builtin_clz(page), pmask = page - 1;
+  const long long page_elems = 2LL * Hkv * page * D;
+  const bf16_t* kbase = cache + (long long)hk * page * D;
+  const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
 
   const int piece = lane % CPR, sub = lane / CPR;
   const bool piece_ok = piece * 8 < D;
@@ -53,9 +58,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     }
   }
 
-  float acc[DEC_DPL];
+  float acc[DPL];
 #pragma unroll
-  for (int i = 0; i < DEC_DPL; ++i) acc[i] = 0.f;
+  for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
   for (int c0 = (lo / DA_WAVE) * DA_WAVE + wave * DA_WAVE; c0 <= p; c0 += DEC_WAVES * DA_WAVE) {
@@ -69,8 +74,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       const int key = c0 + i * G + sub;
       const bool valid = key >= lo && key <= p;
       const int kk = valid ? key : safe_key;
-      const bf16_t* kr = cache + cache_k_row(bt[kk / page], hk, kk % page, Hkv, page, D) + (piece_ok ? piece * 8 : 0);
-      kv[i] = *(const uint4*)kr;
+      kv[i] = *(const uint4*)(kbase + bt[kk >> lg] * page_elems + (kk & pmask) * D + (piece_ok ? piece * 8 : 0));
     }
     const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
     const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
@@ -84,9 +88,12 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
         const int g0 = c0 + g * 8;
         const bool any = g0 + 7 >= first && g0 <= last;
         const int gs = any ? g0 : (last / 8) * 8;
-        vv0[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+        vv0[g] = *(const uint4*)(vbase + bt[gs >> lg] * page_elems + d * page + (gs & pmask));
       }
     }
+    // nothing moves across this line: the compiler would otherwise push the value loads down behind
+    // the scores to save registers, and a chunk would cost a third memory round trip
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
       const int key = c0 + i * G + sub;
@@ -117,9 +124,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     // ---- values: lane owns dimensions lane, lane + 64, ...
 #pragma unroll
-    for (int i = 0; i < DEC_DPL; ++i) {
+    for (int i = 0; i < DPL; ++i) {
       const int d = lane + i * DA_WAVE;
-      if (d >= D) break;
+      if (DPL > 1 && d >= D) break;
       float a = acc[i] * alpha;
       uint4 vv[8];
       if (i == 0) {
@@ -131,23 +138,29 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
           const int g0 = c0 + g * 8;
           const bool any = g0 + 7 >= first && g0 <= last;
           const int gs = any ? g0 : (last / 8) * 8;
-          vv[g] = *(const uint4*)(cache + cache_v_base(bt[gs / page], hk, Hkv, page, D) + (long long)d * page + gs % page);
+          vv[g] = *(const uint4*)(vbase + bt[gs >> lg] * page_elems + d * page + (gs & pmask));
         }
       }
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
+        // Rows outside first..last were never written (or belong to someone else) and may hold anything:
+        // their bits are cleared.  The seen rows of a group are g0+lo8 .. g0+hi8; the masks are the same
+        // for every lane, so the scalar unit builds them.
         const int g0 = c0 + g * 8;
-        const uint32_t u[4] = {vv[g].x, vv[g].y, vv[g].z, vv[g].w};
+        const int lo8 = first - g0 > 0 ? first - g0 : 0, hi8 = last - g0 < 7 ? last - g0 : 7;
+        uint32_t msk[4];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2)
+          msk[e2] = ((2 * e2 >= lo8 && 2 * e2 <= hi8) ? 0x0000ffffu : 0u) |
+                    ((2 * e2 + 1 >= lo8 && 2 * e2 + 1 <= hi8) ? 0xffff0000u : 0u);
+        const uint32_t u[4] = {vv[g].x & msk[0], vv[g].y & msk[1], vv[g].z & msk[2], vv[g].w & msk[3]};
         const float4 w0 = *(const float4*)&ps[wave][g * 8];
         const float4 w1 = *(const float4*)&ps[wave][g * 8 + 4];
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
-          // rows outside first..last were never written (or belong to someone else): keep them out
-          const float v0 = (g0 + 2 * e2 >= first && g0 + 2 * e2 <= last) ? __uint_as_float(u[e2] << 16) : 0.f;
-          const float v1 = (g0 + 2 * e2 + 1 >= first && g0 + 2 * e2 + 1 <= last) ? __uint_as_float(u[e2] & 0xffff0000u) : 0.f;
-          a = fmaf(w[2 * e2], v0, a);
-          a = fmaf(w[2 * e2 + 1], v1, a);
+          a = fmaf(w[2 * e2], __uint_as_float(u[e2] << 16), a);
+          a = fmaf(w[2 * e2 + 1], __uint_as_float(u[e2] & 0xffff0000u), a);
         }
       }
       acc[i] = a;
@@ -157,7 +170,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
 #pragma unroll
-  for (int i = 0; i < DEC_DPL; ++i) {
+  for (int i = 0; i < DPL; ++i) {
     const int d = lane + i * DA_WAVE;
     if (d < D) part_acc[wave][d] = acc[i];
   }
