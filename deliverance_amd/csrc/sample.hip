@@ -193,10 +193,21 @@ sample_kernel(const float* __restrict__ logits, int ldl, int V, const SampleRow*
   const SampleRow sp = params[r];
   const float* row = logits + (size_t)r * ldl;
 
+  // the largest entry (the lowest index among equals): eight loads in flight per thread, from clamped
+  // places, so that the vocabulary is crossed in a few memory round trips
   float best = -INFINITY; int besti = -1;
-  for (int i = threadIdx.x; i < V; i += SAMPLE_THREADS) {
-    const float v = row[i];
-    if (besti < 0 || v > best) { best = v; besti = i; }
+  for (int i0 = threadIdx.x; i0 < V; i0 += 8 * SAMPLE_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      v[u] = row[i < V ? i : V - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      if (i < V && (besti < 0 || v[u] > best)) { best = v[u]; besti = i; }
+    }
   }
   block_best(R, best, besti, false);
   const bool xtc = sp.xtc_threshold != 0.f;
