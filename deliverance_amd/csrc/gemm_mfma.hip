@@ -21,6 +21,7 @@
 // row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
 // l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
 #include "gemm_common.h"
+#include <stdlib.h>
 #include <type_traits>
 
 #define BKT 64               // k per slab
@@ -165,7 +166,7 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
   for (; base + 2 * PF_SLABS <= nslab; base += PF_SLABS) {
     TILE_STEP(0, base, true, true);
     TILE_STEP(1, base + 1, true, true);
-    if (PF_SLABS == 4) {
+    if constexpr (PF_SLABS == 4) {
       TILE_STEP(2, base + 2, true, true);
       TILE_STEP(3, base + 3, true, true);
     }
@@ -173,7 +174,7 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
   for (; base < nslab; base += PF_SLABS) {
     if (base < nslab) TILE_STEP(0, base, base + PF_SLABS < nslab, base + 1 < nslab);
     if (base + 1 < nslab) TILE_STEP(1, base + 1, base + 1 + PF_SLABS < nslab, base + 2 < nslab);
-    if (PF_SLABS == 4) {
+    if constexpr (PF_SLABS == 4) {
       if (base + 2 < nslab) TILE_STEP(2, base + 2, base + 2 + PF_SLABS < nslab, base + 3 < nslab);
       if (base + 3 < nslab) TILE_STEP(3, base + 3, base + 3 + PF_SLABS < nslab, base + 4 < nslab);
     }
@@ -281,8 +282,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
     e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
     e_slot[j] = (ok && kv.cache) ? kv.slot_map[m] : -1;
   }
-  // The wavefront's whole chunks go in groups of SK_UNROLL, then of half that, and so on down to
-  // one: a group is nothing but its loads, all in flight at once, and then its products.  (A value
+  // The wavefront's whole chunks go in groups of SK_UNROLL and one last group of what is left:
+  // a group is nothing but its loads, all in flight at once, and then its products.  (A value
   // replaced after its load, like a zero past K, makes the compiler wait for that load and all
   // before it; that is left to the one chunk that K may cut.)  Rows past M and columns past N read
   // row 0: what they give is never stored.
@@ -307,9 +308,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
     left -= G;
   };
   while (left >= SK_UNROLL) group(std::integral_constant<int, SK_UNROLL>{});
-  if (SK_UNROLL > 4 && left >= 4) group(std::integral_constant<int, 4>{});
-  if (SK_UNROLL > 2 && left >= 2) group(std::integral_constant<int, 2>{});
-  if (left >= 1) group(std::integral_constant<int, 1>{});
+  // what is left goes as one group of exactly that size: one more memory round trip, not several
+  switch (left) {
+    case 7: if (SK_UNROLL > 7) group(std::integral_constant<int, (SK_UNROLL > 7 ? 7 : 1)>{}); break;
+    case 6: if (SK_UNROLL > 6) group(std::integral_constant<int, (SK_UNROLL > 6 ? 6 : 1)>{}); break;
+    case 5: if (SK_UNROLL > 5) group(std::integral_constant<int, (SK_UNROLL > 5 ? 5 : 1)>{}); break;
+    case 4: if (SK_UNROLL > 4) group(std::integral_constant<int, (SK_UNROLL > 4 ? 4 : 1)>{}); break;
+    case 3: if (SK_UNROLL > 3) group(std::integral_constant<int, (SK_UNROLL > 3 ? 3 : 1)>{}); break;
+    case 2: if (SK_UNROLL > 2) group(std::integral_constant<int, (SK_UNROLL > 2 ? 2 : 1)>{}); break;
+    case 1: group(std::integral_constant<int, 1>{}); break;
+    default: break;
+  }
   if (k0 < K) {                                 // the chunk that K cuts (K is a multiple of 8, a chunk is 32 wide)
     const bool kin = k0 + fk < K;
     const int ks = kin ? k0 : -fk;              // a load that is not wanted reads the row's first chunk and is dropped
@@ -388,7 +397,10 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     dim3 grid(da_ceil_div(N, SK_COLS));
     const int mt = da_ceil_div(M, 16);
     // the number of wavefronts that split K depends on K alone, so a row's sums keep their order
-    const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
+    int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
+    static int force_nw = -1;
+    if (force_nw < 0) { const char* e = getenv("DA_SKINNY_NW"); force_nw = e ? atoi(e) : 0; }
+    if (force_nw > 0) nw = force_nw;
     if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
     else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
     else launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
