@@ -270,17 +270,23 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
     arow_ok[i] = r0 + i * 16 + fr < M;
     ap[i] = a + (size_t)(arow_ok[i] ? r0 + i * 16 + fr : 0) * lda + fk;
   }
-  // what the epilogue needs is asked for first, so that it has arrived when the products are done
+  // What the epilogue needs is asked for first, so that it has arrived when the products are done:
+  // as raw bits from places that always exist (a load inside a branch, or a conversion right after
+  // a load, would be waited for here, in front of the loads of the products).
   constexpr int EPT = (MT * 16 * SK_COLS + NW * 64 - 1) / (NW * 64);     // output elements per thread
-  float e_bias[EPT], e_old[EPT];
+  uint32_t e_braw[EPT];
+  float e_old[EPT];
   int e_slot[EPT];
+  const bool bias_bf16 = ep.bias_dtype == DA_BF16;
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = t + j * NW * 64, m = r0 + e / SK_COLS, n = n0 + e % SK_COLS;
     const bool ok = e < MT * 16 * SK_COLS && m < M && n < N;
-    e_bias[j] = (ok && ep.bias) ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
-    e_old[j] = (ok && ep.accumulate) ? ((const float*)ep.out)[(size_t)m * ep.ldo + n] : 0.f;
-    e_slot[j] = (ok && kv.cache) ? kv.slot_map[m] : -1;
+    const void* bsrc = (ok && ep.bias) ? ep.bias : (const void*)w;
+    const int bidx = (ok && ep.bias) ? n : 0;
+    e_braw[j] = bias_bf16 ? (uint32_t)((const bf16_t*)bsrc)[bidx] : ((const uint32_t*)bsrc)[bidx];
+    e_old[j] = *((ok && ep.accumulate) ? (const float*)ep.out + (size_t)m * ep.ldo + n : (const float*)w);
+    e_slot[j] = *((ok && kv.cache) ? kv.slot_map + m : (const int*)w);
   }
   // The wavefront's whole chunks go in groups of SK_UNROLL and one last group of what is left:
   // a group is nothing but its loads, all in flight at once, and then its products.  (A value
@@ -344,7 +350,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
       float v = red[0][ml][c];
 #pragma unroll
       for (int v2 = 1; v2 < NW; ++v2) v += red[v2][ml][c];
-      v = apply_act(v + e_bias[j], ep.act);
+      const float e_bias = !ep.bias ? 0.f : (bias_bf16 ? __uint_as_float(e_braw[j] << 16) : __uint_as_float(e_braw[j]));
+      v = apply_act(v + e_bias, ep.act);
       const size_t o = (size_t)m * ep.ldo + n;
       if (ep.accumulate) ((float*)ep.out)[o] = e_old[j] + v;
       else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);

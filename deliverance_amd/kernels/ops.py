@@ -302,10 +302,11 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     return out
 
 
-# Measured on MI355X inside the model: the fused kernel wins up to 8 rows and a width of 1024 (by
-# 2 to 3 % of a decode step); beyond, the separate norm and product are faster (every 16 output
-# columns recompute the rows' statistics, and a wavefront's loads come in more rounds).
-FUSED_LN_MAX_ROWS = 8
+# Measured on MI355X inside the model: the fused kernel wins up to 16 rows (one row tile) and a
+# width of 1024, by 10 to 15 % of a decode step; beyond, the separate norm and product are faster
+# (every 16 output columns recompute the rows' statistics, and a wavefront's loads come in more
+# rounds).
+FUSED_LN_MAX_ROWS = 16
 FUSED_LN_MAX_K = 1024
 FUSED_LN_MAX_N = 16384      # ... and never for a vocabulary
 FUSED_LN_KERNEL_MAX_ROWS = 32
