@@ -22,7 +22,8 @@
 
 // CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
 template <int CPR, int DEC_WAVES>
-__global__ void __launch_bounds__(DEC_WAVES * DA_WAVE)
+// (registers are held to 128 for head sizes up to 64, so that two workgroups share a compute unit)
+__global__ void __launch_bounds__(DEC_WAVES * DA_WAVE, CPR <= 8 ? 4 : 2)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                    const int* __restrict__ block_table, int max_blocks,
                    const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
@@ -36,27 +37,34 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   const int s = blockIdx.x / Hq, h = blockIdx.x % Hq;
   const int hk = h / (Hq / Hkv);
   const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
-  const int p = seq_lens[s] - 1;                      // the row's position; it sees keys lo..p
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int* bt = block_table + (size_t)s * max_blocks;
   // addressing by shifts: the page size is a power of two (checked on the host)
   const int lg = 31 - __builtin_clz(page), pmask = page - 1;
   const long long page_elems = 2LL * Hkv * page * D;
   const bf16_t* kbase = cache + (long long)hk * page * D;
   const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
-
   const int piece = lane % CPR, sub = lane / CPR;
   const bool piece_ok = piece * 8 < D;
-  float qf[8];
-  {
-    const uint4 qv = *(const uint4*)(q + (size_t)s * q_ld + h * D + (piece_ok ? piece * 8 : 0));
-    const uint32_t u[4] = {qv.x, qv.y, qv.z, qv.w};
+
+  // Asked for before the sequence's length is known, so that they travel beside it: the query (as
+  // raw bits; converted where it is used) and the block-table entries of the chunk this wavefront
+  // starts with when nothing is cut off by a window (keys wave*64 ..).  Entries past the
+  // sequence's pages are read (the table has max_blocks of them) and never used.
+  const uint4 qraw = *(const uint4*)(q + (size_t)s * q_ld + h * D + (piece_ok ? piece * 8 : 0));
+  const int c0_guess = wave * DA_WAVE;
+  int btk0[CPR], btv0[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      qf[2 * e] = piece_ok ? __uint_as_float(u[e] << 16) * scale : 0.f;
-      qf[2 * e + 1] = piece_ok ? __uint_as_float(u[e] & 0xffff0000u) * scale : 0.f;
-    }
+  for (int i = 0; i < CPR; ++i) {
+    const int pg = (c0_guess + i * G + sub) >> lg;
+    btk0[i] = bt[pg < max_blocks ? pg : max_blocks - 1];
   }
+#pragma unroll
+  for (int g = 0; g < 8; ++g) {
+    const int pg = (c0_guess + g * 8) >> lg;
+    btv0[g] = bt[pg < max_blocks ? pg : max_blocks - 1];
+  }
+  const int p = seq_lens[s] - 1;                      // the row's position; it sees keys lo..p
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
 
   float acc[DPL];
 #pragma unroll
@@ -68,18 +76,40 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     // of the weighted sum (both need only the block table), then the arithmetic
     float mine = -INFINITY;      // one key's score per lane, once the loop is done
     uint4 kv[CPR];
-    const int safe_key = p;      // a row that surely exists, read in place of rows that are not seen
+    const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
+    const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
+    // the pages of the chunk's keys and value groups: those asked for at the start, or read now
+    int btk[CPR], btv[8], bt_safe;
+    if (c0 == c0_guess && first == c0) {                 // the same for the whole wavefront
+#pragma unroll
+      for (int i = 0; i < CPR; ++i) btk[i] = btk0[i];
+#pragma unroll
+      for (int g = 0; g < 8; ++g) btv[g] = btv0[g];
+      bt_safe = __builtin_amdgcn_readfirstlane(btk0[0]); // lane 0 holds the page of key c0
+    } else {
+      bt_safe = bt[first >> lg];
+#pragma unroll
+      for (int i = 0; i < CPR; ++i) {
+        const int key = c0 + i * G + sub;
+        btk[i] = bt[((key >= first && key <= last) ? key : first) >> lg];
+      }
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const int g0 = c0 + g * 8;
+        btv[g] = bt[((g0 + 7 >= first && g0 <= last) ? g0 : first) >> lg];
+      }
+    }
+    // a key that is not seen reads `first` instead, a row that surely exists
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
       const int key = c0 + i * G + sub;
       const bool valid = key >= lo && key <= p;
-      const int kk = valid ? key : safe_key;
-      kv[i] = *(const uint4*)(kbase + bt[kk >> lg] * page_elems + (kk & pmask) * D + (piece_ok ? piece * 8 : 0));
+      const long long pg = valid ? btk[i] : bt_safe;
+      const int kk = valid ? key : first;
+      kv[i] = *(const uint4*)(kbase + pg * page_elems + (kk & pmask) * D + (piece_ok ? piece * 8 : 0));
     }
-    const int first = c0 > lo ? c0 : lo;                 // valid keys of the chunk: first..last
-    const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
     // the chunk's 8 groups of 8 keys (a group never crosses a page) of this lane's first dimension;
-    // groups with no seen key read the group of `last` instead and are dropped
+    // groups with no seen key read the group of `first` instead and are dropped
     uint4 vv0[8];
     {
       const int d = lane < D ? lane : 0;
@@ -87,13 +117,23 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       for (int g = 0; g < 8; ++g) {
         const int g0 = c0 + g * 8;
         const bool any = g0 + 7 >= first && g0 <= last;
-        const int gs = any ? g0 : (last / 8) * 8;
-        vv0[g] = *(const uint4*)(vbase + bt[gs >> lg] * page_elems + d * page + (gs & pmask));
+        const int gs = any ? g0 : (first / 8) * 8;
+        const long long pg = any ? btv[g] : bt_safe;
+        vv0[g] = *(const uint4*)(vbase + pg * page_elems + d * page + (gs & pmask));
       }
     }
     // nothing moves across this line: the compiler would otherwise push the value loads down behind
     // the scores to save registers, and a chunk would cost a third memory round trip
     __builtin_amdgcn_sched_barrier(0);
+    float qf[8];
+    {
+      const uint32_t u[4] = {qraw.x, qraw.y, qraw.z, qraw.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        qf[2 * e] = piece_ok ? __uint_as_float(u[e] << 16) * scale : 0.f;
+        qf[2 * e + 1] = piece_ok ? __uint_as_float(u[e] & 0xffff0000u) * scale : 0.f;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
       const int key = c0 + i * G + sub;
@@ -137,8 +177,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
         for (int g = 0; g < 8; ++g) {
           const int g0 = c0 + g * 8;
           const bool any = g0 + 7 >= first && g0 <= last;
-          const int gs = any ? g0 : (last / 8) * 8;
-          vv[g] = *(const uint4*)(vbase + bt[gs >> lg] * page_elems + d * page + (gs & pmask));
+          const int gs = any ? g0 : (first / 8) * 8;
+          const long long pg = any ? btv[g] : bt_safe;
+          vv[g] = *(const uint4*)(vbase + pg * page_elems + d * page + (gs & pmask));
         }
       }
 #pragma unroll
