@@ -111,10 +111,13 @@ __device__ __forceinline__ float4 load_param4(const void* p, int dtype, int i) {
 // once, which is what counts when a step has a handful of rows.  E a multiple of 4, E <= 256*VPL.
 // A workgroup is one wavefront (few rows: as many compute units as rows) or four (many rows: fewer,
 // fuller workgroups).
-template <int VPL>
+// Loads come back in the order they were asked for: the row first, then gain and bias, as raw bits
+// that are converted where they are used (a conversion right after its load, or a load inside a
+// branch, is waited for on the spot).  PBF16: gain and bias are bfloat16 (else 32-bit).
+template <int VPL, bool PBF16>
 __global__ void __launch_bounds__(4 * DA_WAVE)
 layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
-                     const void* __restrict__ w, int w_dtype, const void* __restrict__ b, int b_dtype,
+                     const void* __restrict__ w, const void* __restrict__ b,
                      float eps, void* __restrict__ y, int y_dtype, int R, int E) {
   const int lane = threadIdx.x % DA_WAVE;
   const int r = blockIdx.x * (blockDim.x / DA_WAVE) + threadIdx.x / DA_WAVE;
@@ -122,15 +125,28 @@ layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
   const float* xr = x + (size_t)(rows ? rows[r] : r) * E;
   // every load of the row, of the gain and of the bias is asked for at once (past the row's end
   // the row's start is read and left out of the sums), before anything is reduced
-  float4 v[VPL], g[VPL], bb[VPL];
+  float4 v[VPL];
+  uint4 graw[VPL], braw[VPL];           // bfloat16: .x and .y hold the four values
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
     v[i] = *(const float4*)(xr + (c < E ? c : 0));
-    g[i] = load_param4(w, w_dtype, c < E ? c : 0);
-    bb[i] = b ? load_param4(b, b_dtype, c < E ? c : 0) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
+  const void* bsrc = b ? b : w;         // without a bias the gain is read twice and dropped
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int c = (lane + i * DA_WAVE) * 4, cc = c < E ? c : 0;
+    if (PBF16) {
+      const uint2 g2 = *(const uint2*)((const bf16_t*)w + cc), b2 = *(const uint2*)((const bf16_t*)bsrc + cc);
+      graw[i] = make_uint4(g2.x, g2.y, 0, 0);
+      braw[i] = make_uint4(b2.x, b2.y, 0, 0);
+    } else {
+      graw[i] = *(const uint4*)((const float*)w + cc);
+      braw[i] = *(const uint4*)((const float*)bsrc + cc);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int i = 0; i < VPL; ++i)
     s += ((lane + i * DA_WAVE) * 4 < E ? 1.f : 0.f) * ((v[i].x + v[i].y) + (v[i].z + v[i].w));
@@ -149,8 +165,19 @@ layernorm_row_kernel(const float* __restrict__ x, const int* __restrict__ rows,
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
     if (c < E) {
-      const float4 o = make_float4((v[i].x - mean) * inv * g[i].x + bb[i].x, (v[i].y - mean) * inv * g[i].y + bb[i].y,
-                                   (v[i].z - mean) * inv * g[i].z + bb[i].z, (v[i].w - mean) * inv * g[i].w + bb[i].w);
+      float4 g, bb;
+      if (PBF16) {
+        g = make_float4(__uint_as_float(graw[i].x << 16), __uint_as_float(graw[i].x & 0xffff0000u),
+                        __uint_as_float(graw[i].y << 16), __uint_as_float(graw[i].y & 0xffff0000u));
+        bb = make_float4(__uint_as_float(braw[i].x << 16), __uint_as_float(braw[i].x & 0xffff0000u),
+                         __uint_as_float(braw[i].y << 16), __uint_as_float(braw[i].y & 0xffff0000u));
+      } else {
+        g = make_float4(__uint_as_float(graw[i].x), __uint_as_float(graw[i].y), __uint_as_float(graw[i].z), __uint_as_float(graw[i].w));
+        bb = make_float4(__uint_as_float(braw[i].x), __uint_as_float(braw[i].y), __uint_as_float(braw[i].z), __uint_as_float(braw[i].w));
+      }
+      if (!b) bb = make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 o = make_float4((v[i].x - mean) * inv * g.x + bb.x, (v[i].y - mean) * inv * g.y + bb.y,
+                                   (v[i].z - mean) * inv * g.z + bb.z, (v[i].w - mean) * inv * g.w + bb.w);
       if (y_dtype == DA_BF16) {
         uint2 u;
         u.x = (uint32_t)f32_to_bf16(o.x) | ((uint32_t)f32_to_bf16(o.y) << 16);
@@ -173,10 +200,17 @@ extern "C" int da_layernorm(const float* x, const int* rows, const void* w, int 
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
                        (!b || (uintptr_t)b % 16 == 0);
   const int wpb = R >= 512 ? 4 : 1;      // wavefronts (rows) per workgroup
-  if (E % 4 == 0 && E <= 2048 && aligned) {
-#define LN_LAUNCH(V)                                                                                      \
-  hipLaunchKernelGGL(layernorm_row_kernel<V>, dim3(da_ceil_div(R, wpb)), dim3(wpb * DA_WAVE), 0, st, x, rows, w, \
-                     w_dtype, b, b_dtype, eps, y, y_dtype, R, E)
+  const bool same = (!b || b_dtype == w_dtype) && (w_dtype == DA_BF16 || w_dtype == DA_F32);   // gain and bias alike
+  if (E % 4 == 0 && E <= 2048 && aligned && same) {
+#define LN_LAUNCH(V)                                                                                                \
+  do {                                                                                                              \
+    if (w_dtype == DA_BF16)                                                                                         \
+      hipLaunchKernelGGL((layernorm_row_kernel<V, true>), dim3(da_ceil_div(R, wpb)), dim3(wpb * DA_WAVE), 0, st, x, \
+                         rows, w, b, eps, y, y_dtype, R, E);                                                        \
+    else                                                                                                            \
+      hipLaunchKernelGGL((layernorm_row_kernel<V, false>), dim3(da_ceil_div(R, wpb)), dim3(wpb * DA_WAVE), 0, st, x, \
+                         rows, w, b, eps, y, y_dtype, R, E);                                                        \
+  } while (0)
     if (E <= 256) LN_LAUNCH(1);
     else if (E <= 512) LN_LAUNCH(2);
     else if (E <= 1024) LN_LAUNCH(4);
