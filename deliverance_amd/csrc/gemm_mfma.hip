@@ -21,7 +21,6 @@
 // row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.  16x16x32: lane l gives row / column
 // l % 16 and k = 8 * (l / 16) .. +7; it receives rows 4 * (l / 16) + r, r in 0..3, column l % 16.
 #include "gemm_common.h"
-#include <stdlib.h>
 #include <type_traits>
 
 #define BKT 64               // k per slab
@@ -248,8 +247,9 @@ static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
 // v, v+NW, v+2NW, ... of 32 elements each, several of them in flight at a time.  NW grows with K
 // (fixed by K alone), so that the chain of dependent loads stays short.
 // ---------------------------------------------------------------------------------------------
-#define SK_COLS 16
-template <int MT, int NW, int SK_UNROLL>   // row tiles of 16, wavefronts, k-chunks in flight per wavefront
+// row tiles of 16, wavefronts, k-chunks in flight per wavefront, output columns per workgroup (16, or 8
+// of which the matrix cores' other 8 repeat them and are dropped: twice the workgroups pull on memory)
+template <int MT, int NW, int SK_UNROLL, int SK_COLS>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                    Epilogue ep, KvScatter kv, int M, int N, int K) {
@@ -261,8 +261,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   floatx4 acc[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const bool wrow_ok = n0 + fr < N;
-  const bf16_t* wp = w + (size_t)(wrow_ok ? n0 + fr : 0) * ldw + fk;
+  const int wcol = n0 + fr % SK_COLS;
+  const bf16_t* wp = w + (size_t)(wcol < N ? wcol : 0) * ldw + fk;
   bool arow_ok[MT];
   const bf16_t* ap[MT];
 #pragma unroll
@@ -341,7 +341,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
+    for (int r = 0; r < 4; ++r)
+      if (SK_COLS == 16 || fr < SK_COLS) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
@@ -361,7 +362,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   }
 }
 
-template <int NW>
+template <int NW, int COLS>
 static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
                           const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
   // With few columns the row tiles are spread over more workgroups (blockIdx.y), as long as the chip
@@ -373,10 +374,10 @@ static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int
       break;
     }
   // few rows leave registers for more chunks in flight
-  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
 }
 
 extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
@@ -401,16 +402,19 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
   if (M <= 64) {
-    dim3 grid(da_ceil_div(N, SK_COLS));
     const int mt = da_ceil_div(M, 16);
+    // 8 columns a workgroup where 16 would leave most compute units without one (one row tile only)
+    const int cols = (mt == 1 && da_ceil_div(N, 16) <= 64) ? 8 : 16;
+    dim3 grid(da_ceil_div(N, cols));
     // the number of wavefronts that split K depends on K alone, so a row's sums keep their order
-    int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
-    static int force_nw = -1;
-    if (force_nw < 0) { const char* e = getenv("DA_SKINNY_NW"); force_nw = e ? atoi(e) : 0; }
-    if (force_nw > 0) nw = force_nw;
-    if (nw == 16) launch_skinny<16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else if (nw == 8) launch_skinny<8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else launch_skinny<4>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
+    if (cols == 8) {
+      if (nw == 16) launch_skinny<16, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+      else if (nw == 8) launch_skinny<8, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+      else launch_skinny<4, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    } else if (nw == 16) launch_skinny<16, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else if (nw == 8) launch_skinny<8, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    else launch_skinny<4, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
   } else {
     // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
     // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so
