@@ -23,7 +23,7 @@
 // CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
 template <int CPR, int DEC_WAVES>
 // (registers are held to 128 for head sizes up to 64, so that two workgroups share a compute unit)
-__global__ void __launch_bounds__(DEC_WAVES * DA_WAVE, CPR <= 8 ? 4 : 2)
+__global__ void __launch_bounds__(DEC_WAVES * DA_WAVE, (CPR <= 8 || DEC_WAVES == 16) ? 4 : 2)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                    const int* __restrict__ block_table, int max_blocks,
                    const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
@@ -250,14 +250,16 @@ extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const 
              "attn_decode: q and the cache must be 16-byte aligned");
   if (S == 0) return 0;
   const int pieces = D / 8;
-  // 8 wavefronts: 16 cost more to start than they hide, 4 leave a context of 1,024 two chunks deep
+  // 8 wavefronts; 16 where the workgroups are few (a context above 512 is then still one chunk a
+  // wavefront, and the larger workgroup's start is paid once per compute unit)
+  const bool wide = (long)S * Hq <= 128 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
   dim3 grid(S * Hq);
   hipStream_t st = (hipStream_t)stream;
 #define LAUNCH2(C, W)                                                                                      \
   hipLaunchKernelGGL((attn_decode_kernel<C, W>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld,   \
                      (const bf16_t*)cache, block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, \
                      (bf16_t*)out, out_ld)
-#define LAUNCH(C) LAUNCH2(C, 8)
+#define LAUNCH(C) do { if (wide) LAUNCH2(C, 16); else LAUNCH2(C, 8); } while (0)
   if (pieces <= 2) LAUNCH(2);
   else if (pieces <= 4) LAUNCH(4);
   else if (pieces <= 8) LAUNCH(8);
