@@ -406,7 +406,8 @@ def test_xtc_and_logprobs(ops):
 
 
 # ----------------------------------------------------------------------------- fused norm + product
-@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 2304, 768), (17, 1000, 96), (32, 200, 1600), (5, 50257, 768)])
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 2304, 768), (17, 1000, 96), (32, 200, 1600), (5, 50257, 768),
+                                   (16, 520, 1024), (12, 72, 1000), (9, 40, 520)])
 @pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_product(ops, M, N, K, pdtype):
     g = torch.Generator().manual_seed(M + N)
