@@ -145,8 +145,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
         dot = fmaf(qf[2 * e], __uint_as_float(u[e] << 16), dot);
         dot = fmaf(qf[2 * e + 1], __uint_as_float(u[e] & 0xffff0000u), dot);
       }
-#pragma unroll
-      for (int o = 1; o < CPR; o <<= 1) dot += __shfl_xor(dot, o, DA_WAVE);
+      dot = group_sum<CPR>(dot);
       // all CPR lanes of the group now hold the score; the lane whose piece number is i keeps it
       if (piece == i) mine = valid ? dot : -INFINITY;
     }

@@ -83,16 +83,44 @@ __device__ __forceinline__ void store_out(void* p, int dtype, size_t i, float v)
   else ((float*)p)[i] = v;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = DA_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, DA_WAVE);
+// Reductions over the wavefront by DPP moves fused into the additions (a lane exchange through
+// __shfl_xor goes through LDS hardware and costs about twenty times as much).  Every lane must be
+// active.  quad_perm [1,0,3,2] and [2,3,0,1] add the lanes of a quad, row_half_mirror the two quads
+// of eight lanes, row_mirror the two halves of a row of 16; row_bcast:15 and :31 carry the rows'
+// totals up to lane 63, which is then read for all.  The order of the additions is fixed.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v),
+                                                               CTRL, ROWMASK, 0xF, false));
+}
+
+// the sum over groups of N consecutive lanes (N a power of two), in every lane of the group
+template <int N>
+__device__ __forceinline__ float group_sum(float v) {
+  if (N >= 2) v += dpp_move<0xB1, 0xF>(0.f, v);
+  if (N >= 4) v += dpp_move<0x4E, 0xF>(0.f, v);
+  if (N >= 8) v += dpp_move<0x141, 0xF>(0.f, v);
+  if (N >= 16) v += dpp_move<0x140, 0xF>(0.f, v);
+  if (N >= 32) v += __shfl_xor(v, 16, DA_WAVE);
+  if (N >= 64) v += __shfl_xor(v, 32, DA_WAVE);
   return v;
 }
 
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group_sum<16>(v);
+  v += dpp_move<0x142, 0xA>(0.f, v);        // rows 1 and 3 take the total of the row before
+  v += dpp_move<0x143, 0xC>(0.f, v);        // rows 2 and 3 take lane 31's: row 3 now holds all four
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), DA_WAVE - 1));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = DA_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, DA_WAVE));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x4E, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x141, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x140, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x142, 0xA>(v, v));
+  v = fmaxf(v, dpp_move<0x143, 0xC>(v, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), DA_WAVE - 1));
 }
 
 // A workgroup barrier that orders LDS traffic only: loads from global memory that were issued
