@@ -113,6 +113,57 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), DA_WAVE - 1));
 }
 
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ int dpp_move_i(int old, int v) {
+  return __builtin_amdgcn_update_dpp(old, v, CTRL, ROWMASK, 0xF, false);
+}
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ double dpp_move_d(double old, double v) {
+  const long long o = __builtin_bit_cast(long long, old), x = __builtin_bit_cast(long long, v);
+  const unsigned lo = (unsigned)dpp_move_i<CTRL, ROWMASK>((int)o, (int)x);
+  const unsigned hi = (unsigned)dpp_move_i<CTRL, ROWMASK>((int)(o >> 32), (int)(x >> 32));
+  return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+}
+
+__device__ __forceinline__ int wave_sum_i(int v) {
+  v += dpp_move_i<0xB1, 0xF>(0, v);
+  v += dpp_move_i<0x4E, 0xF>(0, v);
+  v += dpp_move_i<0x141, 0xF>(0, v);
+  v += dpp_move_i<0x140, 0xF>(0, v);
+  v += dpp_move_i<0x142, 0xA>(0, v);
+  v += dpp_move_i<0x143, 0xC>(0, v);
+  return __builtin_amdgcn_readlane(v, DA_WAVE - 1);
+}
+
+__device__ __forceinline__ double wave_sum_d(double v) {
+  v += dpp_move_d<0xB1, 0xF>(0.0, v);
+  v += dpp_move_d<0x4E, 0xF>(0.0, v);
+  v += dpp_move_d<0x141, 0xF>(0.0, v);
+  v += dpp_move_d<0x140, 0xF>(0.0, v);
+  v += dpp_move_d<0x142, 0xA>(0.0, v);
+  v += dpp_move_d<0x143, 0xC>(0.0, v);
+  const long long x = __builtin_bit_cast(long long, v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)x, DA_WAVE - 1);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(x >> 32), DA_WAVE - 1);
+  return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+}
+
+// The best (value, index) pair of the wavefront under `better(a, ai, b, bi)` (a strict order), in every lane.
+template <class Better>
+__device__ __forceinline__ void wave_best(float& v, int& idx, Better better) {
+#define DA_BEST_STEP(CTRL, ROWMASK)                                   \
+  {                                                                   \
+    const float ov = dpp_move<CTRL, ROWMASK>(v, v);                   \
+    const int oi = dpp_move_i<CTRL, ROWMASK>(idx, idx);               \
+    if (better(ov, oi, v, idx)) { v = ov; idx = oi; }                 \
+  }
+  DA_BEST_STEP(0xB1, 0xF) DA_BEST_STEP(0x4E, 0xF) DA_BEST_STEP(0x141, 0xF) DA_BEST_STEP(0x140, 0xF)
+  DA_BEST_STEP(0x142, 0xA) DA_BEST_STEP(0x143, 0xC)
+#undef DA_BEST_STEP
+  v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), DA_WAVE - 1));
+  idx = __builtin_amdgcn_readlane(idx, DA_WAVE - 1);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp_move<0xB1, 0xF>(v, v));
   v = fmaxf(v, dpp_move<0x4E, 0xF>(v, v));

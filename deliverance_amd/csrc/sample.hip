@@ -45,11 +45,8 @@ struct Reducer {
 };
 
 __device__ void block_sum(const Reducer& R, double& mass, int& count) {
-#pragma unroll
-  for (int o = DA_WAVE / 2; o > 0; o >>= 1) {
-    mass += __shfl_xor(mass, o, DA_WAVE);
-    count += __shfl_xor(count, o, DA_WAVE);
-  }
+  mass = wave_sum_d(mass);
+  count = wave_sum_i(count);
   const int wave = threadIdx.x / DA_WAVE, lane = threadIdx.x % DA_WAVE;
   __syncthreads();
   if (lane == 0) { R.d[wave] = mass; R.i[wave] = count; }
@@ -68,12 +65,7 @@ __device__ void block_best(const Reducer& R, float& v, int& idx, bool want_min) 
     if (a != b) return want_min ? a < b : a > b;
     return ai < bi;
   };
-#pragma unroll
-  for (int o = DA_WAVE / 2; o > 0; o >>= 1) {
-    float ov = __shfl_xor(v, o, DA_WAVE);
-    int oi = __shfl_xor(idx, o, DA_WAVE);
-    if (better(ov, oi, v, idx)) { v = ov; idx = oi; }
-  }
+  wave_best(v, idx, better);
   const int wave = threadIdx.x / DA_WAVE, lane = threadIdx.x % DA_WAVE;
   __syncthreads();
   if (lane == 0) { R.f[wave] = v; R.i[wave] = idx; }
