@@ -5,6 +5,7 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4s_t;   // the 4x4x4 form takes its bfloat16 as shorts
 
 struct Epilogue {
   const void* bias;

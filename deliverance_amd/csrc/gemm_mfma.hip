@@ -3,7 +3,7 @@
 //   out[m, n] (+)= act( sum_k a[m, k] * w[n, k] + bias[n] )
 //
 // a: [M, K] bf16, w: [N, K] bf16 ("[out, in]", K contiguous), 32-bit accumulation; out is bf16,
-// or 32-bit (plain store or += for the residual stream).  Two kernels:
+// or 32-bit (plain store or += for the residual stream).  Three kernels:
 //
 //  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
 //    buffers, with the next four slabs already in flight in registers.  For steps with many rows
@@ -12,8 +12,10 @@
 //    columns, some of the 16-row tiles); its
 //    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
 //    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
+//  * gemm_skinny4: for M <= 16 and up to 2,048 columns (decode's out-proj and proj).  MFMA 4x4x4, whose
+//    operand layout lets a row of w be read in whole cache lines; 4 or 8 columns a workgroup.
 //
-// In both, an output element sums over k in an order that depends on K only, never on M or on
+// In each, an output element sums over k in an order that depends on K only, never on M or on
 // the row's place in the batch.
 //
 // MFMA fragment layout (64 lanes).  32x32x16: lane l gives row (a) / column (b) l % 32 and the
@@ -362,6 +364,160 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// M <= 16.  MFMA 4x4x4: 16 independent 4x4 products of depth 4 a wavefront.  Lane l gives row (a) /
+// column (b) l % 4 of product l / 4 and 4 consecutive k; it receives column l % 4 of that product,
+// rows 0..3.  The 16 products of a step take 16 consecutive pieces of k of 8 elements (two
+// instructions each), so a lane loads 16 bytes and the 16 lanes of one row of w read 256 consecutive
+// bytes: whole cache lines.  (The 16x16x32 form reads 16 rows x 64 bytes a load, and a compute unit's
+// L1 passes that at a third of the rate.)  A workgroup owns 4 * NG columns; wavefront v of NW takes
+// the steps v, v+NW, ... of 128 elements of k; the products of a wavefront are summed over its 16
+// lanes-groups at the end (two lane rotations, then LDS) in a fixed order.
+// ---------------------------------------------------------------------------------------------
+template <int MG, int NG, int NW, int UNROLL>
+__global__ void __launch_bounds__(NW * 64)
+gemm_skinny4_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
+                    Epilogue ep, KvScatter kv, int M, int N, int K) {
+  constexpr int ROWS = MG * 4, COLS = NG * 4;
+  __shared__ __attribute__((aligned(16))) float red[4 * NW][COLS][ROWS];
+  static_assert(NW * 64 >= 4 * ROWS * COLS, "four threads an output element");
+  const int t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int n0 = blockIdx.x * COLS;
+  const int q = lane % 4, kb = (lane / 4) * 8;
+  const bf16_t* wp[NG];
+  const bf16_t* ap[MG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int n = n0 + g * 4 + q;
+    wp[g] = w + (size_t)(n < N ? n : 0) * ldw + kb;
+  }
+#pragma unroll
+  for (int g = 0; g < MG; ++g) {
+    const int m = g * 4 + q;
+    ap[g] = a + (size_t)(m < M ? m : 0) * lda + kb;
+  }
+  // what the epilogue needs is asked for first, as raw bits from places that always exist
+  // Four threads an output element (the host launches 4 * ROWS * COLS threads at least): each sums
+  // a quarter of the partial sums, the first of them stores.
+  const int e_id = t / 4, e_q = t % 4;
+  const int e_m = e_id / COLS, e_c = e_id % COLS, e_n = n0 + e_c;
+  const bool e_ok = e_id < ROWS * COLS && e_m < M && e_n < N;
+  const bool e_st = e_ok && e_q == 0;
+  const bool bias_bf16 = ep.bias_dtype == DA_BF16;
+  const void* e_bsrc = (e_st && ep.bias) ? ep.bias : (const void*)w;
+  const int e_bidx = (e_st && ep.bias) ? e_n : 0;
+  const uint32_t e_braw = bias_bf16 ? (uint32_t)((const bf16_t*)e_bsrc)[e_bidx] : ((const uint32_t*)e_bsrc)[e_bidx];
+  const float e_old = *((e_st && ep.accumulate) ? (const float*)ep.out + (size_t)e_m * ep.ldo + e_n : (const float*)w);
+  const int e_slot = *((e_st && kv.cache) ? kv.slot_map + e_m : (const int*)w);
+
+  floatx4 acc[MG][NG];
+#pragma unroll
+  for (int i = 0; i < MG; ++i)
+#pragma unroll
+    for (int j = 0; j < NG; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // The wavefront's steps go in groups of UNROLL and one last group of what is left: a group is
+  // nothing but its loads, all in flight at once, and then its products.  The last step of the last
+  // group may be the one that K cuts: lanes past K read the row's first piece instead and give
+  // zeros for a (a multiple of 8 elements is in or out as a whole).
+  const int steps = (K + 127) / 128;
+  int count = wave < steps ? (steps - wave + NW - 1) / NW : 0;
+  int k0 = wave * 128;
+  auto group = [&](auto gc, auto lastc) {
+    constexpr int G = decltype(gc)::value;
+    constexpr bool LAST = decltype(lastc)::value;
+    uint4 av[G][MG], wv[G][NG];
+    bool kin = true;
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+      int kk = k0 + u * NW * 128;
+      if (LAST && u == G - 1) {
+        kin = kk + kb < K;
+        kk = kin ? kk : -kb;
+      }
+#pragma unroll
+      for (int i = 0; i < MG; ++i) av[u][i] = load16(ap[i] + kk);
+#pragma unroll
+      for (int j = 0; j < NG; ++j) wv[u][j] = load16(wp[j] + kk);
+    }
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+      if (LAST && u == G - 1) {
+#pragma unroll
+        for (int i = 0; i < MG; ++i)
+          if (!kin) av[u][i] = make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < MG; ++i)
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+              __builtin_bit_cast(bf16x4s_t, make_uint2(av[u][i].x, av[u][i].y)),
+              __builtin_bit_cast(bf16x4s_t, make_uint2(wv[u][j].x, wv[u][j].y)), acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+              __builtin_bit_cast(bf16x4s_t, make_uint2(av[u][i].z, av[u][i].w)),
+              __builtin_bit_cast(bf16x4s_t, make_uint2(wv[u][j].z, wv[u][j].w)), acc[i][j], 0, 0, 0);
+        }
+    }
+    k0 += G * NW * 128;
+    count -= G;
+  };
+  while (count > UNROLL) group(std::integral_constant<int, UNROLL>{}, std::false_type{});
+  switch (count) {
+    case 4: if (UNROLL >= 4) group(std::integral_constant<int, (UNROLL >= 4 ? 4 : 1)>{}, std::true_type{}); break;
+    case 3: if (UNROLL >= 3) group(std::integral_constant<int, (UNROLL >= 3 ? 3 : 1)>{}, std::true_type{}); break;
+    case 2: if (UNROLL >= 2) group(std::integral_constant<int, (UNROLL >= 2 ? 2 : 1)>{}, std::true_type{}); break;
+    case 1: group(std::integral_constant<int, 1>{}, std::true_type{}); break;
+    default: break;
+  }
+  // sum over the four products of a row of 16 lanes, then one partial a row of lanes goes to LDS
+#pragma unroll
+  for (int i = 0; i < MG; ++i)
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      floatx4 v = acc[i][j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] += dpp_move<0x124, 0xF>(v[r], v[r]);      // row_ror:4
+        v[r] += dpp_move<0x128, 0xF>(v[r], v[r]);      // row_ror:8
+      }
+      if (lane % 16 < 4) *(floatx4*)&red[wave * 4 + lane / 16][j * 4 + q][i * 4] = v;
+    }
+  lds_barrier();
+  if (e_id < ROWS * COLS) {               // whole quads
+    // thread e_q of the four takes the partial sums e_q, e_q + 4, ...: one of each wavefront
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) v += red[e_q + 4 * i][e_c][e_m];
+    v += dpp_move<0xB1, 0xF>(v, v);
+    v += dpp_move<0x4E, 0xF>(v, v);
+    if (e_st) {
+      const float e_bias = !ep.bias ? 0.f : (bias_bf16 ? __uint_as_float(e_braw << 16) : __uint_as_float(e_braw));
+      v = apply_act(v + e_bias, ep.act);
+      const size_t o = (size_t)e_m * ep.ldo + e_n;
+      if (ep.accumulate) ((float*)ep.out)[o] = e_old + v;
+      else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
+      else ((float*)ep.out)[o] = v;
+      if (kv.cache && e_n >= kv.q_cols && e_slot >= 0) kv_scatter_store(kv, e_slot, e_n, v);
+    }
+  }
+}
+
+template <int MG, int NG>
+static int launch_skinny4(int nw, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
+                          const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
+  static_assert(MG * NG <= 8, "four threads an output element in 16 wavefronts at most");
+  DA_REQUIRE(M <= MG * 4, "gemm_bf16: %d rows for %d groups of 4", M, MG);
+  const dim3 grid(da_ceil_div(N, NG * 4));
+  constexpr int U = MG + NG <= 4 ? 4 : (MG + NG <= 6 ? 3 : 2);
+  // (4 wavefronts are too few threads for 8 groups: 8 then)
+#define DA_SK4_GO(NWv) hipLaunchKernelGGL((gemm_skinny4_kernel<MG, NG, (NWv < MG * NG ? 8 : NWv), U>), grid, dim3((NWv < MG * NG ? 8 : NWv) * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K)
+  if (nw > 8) DA_SK4_GO(16);
+  else if (nw > 4) DA_SK4_GO(8);
+  else DA_SK4_GO(4);
+#undef DA_SK4_GO
+  return 0;
+}
+
 template <int NW, int COLS>
 static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
                           const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
@@ -401,7 +557,20 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
-  if (M <= 64) {
+  if (M <= 16 && N <= 2048 && (M <= 8 || K >= 2048)) {
+    // Measured: the 4x4x4 form wins where few workgroups pull on memory (up to 2,048 columns; by 25 to 40 %
+    // with K from 2,048 on).  With more columns both forms stream alike and the other one's sums are cheaper;
+    // beyond 8 rows the loads of a outweigh it unless K is large.
+    const int mg = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
+    const int ng = N <= 1024 ? 1 : 2;
+    const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // by K alone, so a row's sums keep their order
+#define DA_SK4(MG, NG) launch_skinny4<MG, NG>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)
+    int rc;
+    if (ng == 1) rc = mg == 1 ? DA_SK4(1, 1) : (mg == 2 ? DA_SK4(2, 1) : DA_SK4(4, 1));
+    else rc = mg == 1 ? DA_SK4(1, 2) : (mg == 2 ? DA_SK4(2, 2) : DA_SK4(4, 2));
+    if (rc) return rc;
+#undef DA_SK4
+  } else if (M <= 64) {
     const int mt = da_ceil_div(M, 16);
     // 8 columns a workgroup where 16 would leave most compute units without one (one row tile only)
     const int cols = (mt == 1 && da_ceil_div(N, 16) <= 64) ? 8 : 16;

@@ -99,9 +99,11 @@ def test_gemm_plain_32bit(ops, M, N, K):
         assert (out - ref).abs().max() < 2e-5 * max(1.0, ref.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [1, 3, 16, 17, 40, 64, 65, 128, 200, 513])
-@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24)])
+@pytest.mark.parametrize("M", [1, 3, 5, 8, 12, 16, 17, 40, 64, 65, 128, 200, 513])
+@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24), (300, 2056), (1030, 1160)])
 def test_gemm_matrix_cores(ops, M, N, K):
+    """Every kernel form behind ``linear_mfma`` (few rows and few columns: 4x4x4 products with 1, 2 or 4
+    row groups, 4 to 16 wavefronts, a last step that K cuts; few rows: 16x16x32; else block tiles)."""
     g = torch.Generator().manual_seed(M * 7 + N)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
                                (None, True, True, torch.float32), (None, False, False, torch.float32),
@@ -112,21 +114,30 @@ def test_gemm_matrix_cores(ops, M, N, K):
 
 
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
-    """A row's result is the same whatever other rows share the call (within one kernel)."""
+    """A row's result is the same, bit for bit, whatever other rows share the call, as long as the call
+    takes the same kernel form (block tiles; 16x16x32 products for 9 to 64 rows; 4x4x4 products up to 8
+    rows and 2,048 columns); between forms it differs by the rounding of 32-bit sums at most."""
     g = torch.Generator().manual_seed(3)
     K, N = 768, 300
     a = bf(torch.randn(200, K, generator=g)).to(DEV)
     w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
-    full = torch.empty(200, N, device=DEV, dtype=torch.bfloat16)
-    ops.linear_mfma(a, w, None, full)
-    part = torch.empty(90, N, device=DEV, dtype=torch.bfloat16)
-    ops.linear_mfma(a[60:150].contiguous(), w, None, part)
-    assert torch.equal(part, full[60:150])
-    small = torch.empty(64, N, device=DEV, dtype=torch.bfloat16)
-    ops.linear_mfma(a[:64].contiguous(), w, None, small)
-    one = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
-    ops.linear_mfma(a[10:11].contiguous(), w, None, one)
-    assert torch.equal(one[0], small[10])
+
+    def rows(lo, hi, dtype=torch.bfloat16):
+        out = torch.empty(hi - lo, N, device=DEV, dtype=dtype)
+        ops.linear_mfma(a[lo:hi].contiguous(), w, None, out)
+        return out
+
+    full = rows(0, 200)
+    assert torch.equal(rows(60, 150), full[60:150])                 # block tiles
+    small = rows(0, 64)
+    assert torch.equal(rows(3, 23)[7], small[10])                   # 16x16x32: 20 rows, 64 rows
+    assert torch.equal(rows(10, 11)[0], rows(4, 12)[6])             # 4x4x4: 1 row, 8 rows
+    assert torch.equal(rows(10, 13)[0], rows(10, 11)[0])            # ... 3 rows
+    exact = a[10].double() @ w.double().t()
+    scale = exact.abs().max().item()
+    forms = [rows(10, 11, torch.float32)[0], rows(0, 64, torch.float32)[10], rows(0, 200, torch.float32)[10]]
+    for f in forms:
+        assert (f.double() - exact).abs().max() < 2e-6 * scale
 
 
 def test_gemm_refuses_what_it_cannot_take(ops):
