@@ -8,12 +8,11 @@
 //  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
 //    buffers, with the next four slabs already in flight in registers.  For steps with many rows
 //    (prefill).
-//  * gemm_skinny: for M <= 64 (decode).  One block owns 16 output columns and all rows (or, with few
-//    columns, some of the 16-row tiles); its
-//    wavefronts (4 to 16, by K) split K, stream their part of w straight from memory into MFMA 16x16x32
-//    fragments and reduce through LDS in a fixed order.  Bound by the bytes of w.
-//  * gemm_skinny4: for M <= 16 and up to 2,048 columns (decode's out-proj and proj).  MFMA 4x4x4, whose
-//    operand layout lets a row of w be read in whole cache lines; 4 or 8 columns a workgroup.
+//  * gemm_skinny: for M <= 64 (decode).  A workgroup owns 16 output columns; its wavefronts (4 to 12)
+//    split K, pull their part of a and w from memory in whole cache lines, pass it through LDS into
+//    MFMA 16x16x32 fragments and add their sums through LDS in a fixed order.  Bound by the bytes of w.
+//  * gemm_skinny4: for M <= 4 and up to 2,048 columns.  MFMA 4x4x4, whose operand layout lets a row
+//    of w be read in whole cache lines straight into registers; 4 or 8 columns a workgroup.
 //
 // In each, an output element sums over k in an order that depends on K only, never on M or on
 // the row's place in the batch.
@@ -245,111 +244,136 @@ static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
 }
 
 // ---------------------------------------------------------------------------------------------
-// M <= 64.  Block: 16 columns of the output, all rows; wavefront v of NW takes the k-chunks
-// v, v+NW, v+2NW, ... of 32 elements each, several of them in flight at a time.  NW grows with K
-// (fixed by K alone), so that the chain of dependent loads stays short.
+// M <= 64.  A workgroup owns 16 output columns and MT row tiles of 16 (all of them, or with few
+// columns some: blockIdx.y); wavefront v of NW takes the steps v, v+NW, ... of 64 elements of k, so
+// that NW chains of loads run side by side; MFMA 16x16x32; the wavefronts' sums are added through
+// LDS in a fixed order.  The operands come in whole cache lines: a load takes 8 rows x 128 bytes,
+// the wavefront parks a step in its own piece of LDS and reads the fragments from there.  (Loaded
+// straight in fragment order, 16 rows x 64 bytes a load, they pass a compute unit's L1 at a third
+// of the rate, and that rate, not the memory's, bounds a workgroup.)
 // ---------------------------------------------------------------------------------------------
-// row tiles of 16, wavefronts, k-chunks in flight per wavefront, output columns per workgroup (16, or 8
-// of which the matrix cores' other 8 repeat them and are dropped: twice the workgroups pull on memory)
-template <int MT, int NW, int SK_UNROLL, int SK_COLS>
+#define SK_LD (64 + 8)       // padded row of a step in LDS, elements (144 bytes)
+template <int MT, int NW, int UNROLL>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                   Epilogue ep, KvScatter kv, int M, int N, int K) {
-  __shared__ float red[NW][MT * 16][SK_COLS + 1];
+                       Epilogue ep, KvScatter kv, int M, int N, int K) {
+  constexpr int AR = MT * 16, TR = AR + 16;          // rows of a; rows of a step: a's, then w's 16
+  constexpr int AL = MT * 2;                         // loads of 8 rows that cover a
+  // the wavefronts' partial sums take the place of the parked steps once all products are done
+  constexpr int STAGE_BYTES = NW * TR * SK_LD * 2, RED_BYTES = NW * AR * 17 * 4;
+  __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES];
+  bf16_t (*stage)[TR * SK_LD] = (bf16_t (*)[TR * SK_LD])smem;
+  float (*red)[AR][17] = (float (*)[AR][17])smem;
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
-  const int n0 = blockIdx.x * SK_COLS;
-  const int r0 = blockIdx.y * MT * 16;             // the workgroup's first row
-  const int fr = lane % 16, fk = (lane / 16) * 8;
-  floatx4 acc[MT];
+  const int n0 = blockIdx.x * 16;
+  const int r0 = blockIdx.y * AR;                    // the workgroup's first row
+  const int lr = lane / 8, lc = (lane % 8) * 8;      // a load: row lr of 8, 16-byte piece lane % 8
+  const int fr = lane % 16, fk = (lane / 16) * 8;    // a fragment: row fr of 16, k-group lane / 16
+  const bf16_t* pa[AL];
+  const bf16_t* pw[2];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int wcol = n0 + fr % SK_COLS;
-  const bf16_t* wp = w + (size_t)(wcol < N ? wcol : 0) * ldw + fk;
-  bool arow_ok[MT];
-  const bf16_t* ap[MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    arow_ok[i] = r0 + i * 16 + fr < M;
-    ap[i] = a + (size_t)(arow_ok[i] ? r0 + i * 16 + fr : 0) * lda + fk;
+  for (int i = 0; i < AL; ++i) {
+    const int m = r0 + i * 8 + lr;
+    pa[i] = a + (size_t)(m < M ? m : 0) * lda + lc;
   }
-  // What the epilogue needs is asked for first, so that it has arrived when the products are done:
-  // as raw bits from places that always exist (a load inside a branch, or a conversion right after
-  // a load, would be waited for here, in front of the loads of the products).
-  constexpr int EPT = (MT * 16 * SK_COLS + NW * 64 - 1) / (NW * 64);     // output elements per thread
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int n = n0 + i * 8 + lr;
+    pw[i] = w + (size_t)(n < N ? n : 0) * ldw + lc;
+  }
+  // what the epilogue needs is asked for first, as raw bits from places that always exist
+  constexpr int EPT = (AR * 16 + NW * 64 - 1) / (NW * 64);
   uint32_t e_braw[EPT];
   float e_old[EPT];
   int e_slot[EPT];
   const bool bias_bf16 = ep.bias_dtype == DA_BF16;
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, m = r0 + e / SK_COLS, n = n0 + e % SK_COLS;
-    const bool ok = e < MT * 16 * SK_COLS && m < M && n < N;
+    const int e = t + j * NW * 64, m = r0 + e / 16, n = n0 + e % 16;
+    const bool ok = e < AR * 16 && m < M && n < N;
     const void* bsrc = (ok && ep.bias) ? ep.bias : (const void*)w;
     const int bidx = (ok && ep.bias) ? n : 0;
     e_braw[j] = bias_bf16 ? (uint32_t)((const bf16_t*)bsrc)[bidx] : ((const uint32_t*)bsrc)[bidx];
     e_old[j] = *((ok && ep.accumulate) ? (const float*)ep.out + (size_t)m * ep.ldo + n : (const float*)w);
     e_slot[j] = *((ok && kv.cache) ? kv.slot_map + m : (const int*)w);
   }
-  // The wavefront's whole chunks go in groups of SK_UNROLL and one last group of what is left:
-  // a group is nothing but its loads, all in flight at once, and then its products.  (A value
-  // replaced after its load, like a zero past K, makes the compiler wait for that load and all
-  // before it; that is left to the one chunk that K may cut.)  Rows past M and columns past N read
-  // row 0: what they give is never stored.
-  int k0 = wave * 32;
-  int left = k0 + 32 <= K ? (K - 32 - k0) / (NW * 32) + 1 : 0;        // whole chunks of this wavefront
-  auto group = [&](auto gc) {
+  floatx4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16_t* mine = stage[wave];
+  // The wavefront's steps (v, v+NW, ...) go two at a time: all loads of both first, then each is
+  // parked in LDS and multiplied.  The very last step may be the one that K cuts: lanes past K read
+  // the row's first piece instead and park zeros.
+  const int steps = (K + 63) / 64;
+  int count = wave < steps ? (steps - wave + NW - 1) / NW : 0;
+  int k0 = wave * 64;
+  auto group = [&](auto gc, auto lastc) {
     constexpr int G = decltype(gc)::value;
-    uint4 wv[G], av[G][MT];
+    constexpr bool LAST = decltype(lastc)::value;
+    uint4 av[G][AL], wv[G][2];
+    bool kin = true;
 #pragma unroll
     for (int u = 0; u < G; ++u) {
-      wv[u] = load16(wp + k0 + u * NW * 32);
+      int kk = k0 + u * NW * 64;
+      if (LAST && u == G - 1) {
+        kin = kk + lc < K;
+        kk = kin ? kk : -lc;
+      }
 #pragma unroll
-      for (int i = 0; i < MT; ++i) av[u][i] = load16(ap[i] + k0 + u * NW * 32);
+      for (int i = 0; i < AL; ++i) av[u][i] = load16(pa[i] + kk);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) wv[u][i] = load16(pw[i] + kk);
     }
 #pragma unroll
-    for (int u = 0; u < G; ++u)
+    for (int u = 0; u < G; ++u) {
 #pragma unroll
-      for (int i = 0; i < MT; ++i)
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u][i]),
-                                                         __builtin_bit_cast(bf16x8_t, wv[u]), acc[i], 0, 0, 0);
-    k0 += G * NW * 32;
-    left -= G;
+      for (int i = 0; i < AL; ++i) *(uint4*)&mine[(i * 8 + lr) * SK_LD + lc] = av[u][i];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = wv[u][i];
+      if (LAST && u == G - 1 && !kin) {        // past K: zeros over what the lane just parked
+        const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < AL; ++i) *(uint4*)&mine[(i * 8 + lr) * SK_LD + lc] = zero;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = zero;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#pragma unroll
+      for (int c = 0; c < 64; c += 32) {
+        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[(AR + fr) * SK_LD + c + fk]);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[(i * 16 + fr) * SK_LD + c + fk]);
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc[i], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+    k0 += G * NW * 64;
+    count -= G;
   };
-  while (left >= SK_UNROLL) group(std::integral_constant<int, SK_UNROLL>{});
-  // what is left goes as one group of exactly that size: one more memory round trip, not several
-  switch (left) {
-    case 7: if (SK_UNROLL > 7) group(std::integral_constant<int, (SK_UNROLL > 7 ? 7 : 1)>{}); break;
-    case 6: if (SK_UNROLL > 6) group(std::integral_constant<int, (SK_UNROLL > 6 ? 6 : 1)>{}); break;
-    case 5: if (SK_UNROLL > 5) group(std::integral_constant<int, (SK_UNROLL > 5 ? 5 : 1)>{}); break;
-    case 4: if (SK_UNROLL > 4) group(std::integral_constant<int, (SK_UNROLL > 4 ? 4 : 1)>{}); break;
-    case 3: if (SK_UNROLL > 3) group(std::integral_constant<int, (SK_UNROLL > 3 ? 3 : 1)>{}); break;
-    case 2: if (SK_UNROLL > 2) group(std::integral_constant<int, (SK_UNROLL > 2 ? 2 : 1)>{}); break;
-    case 1: group(std::integral_constant<int, 1>{}); break;
+  while (count > UNROLL) group(std::integral_constant<int, UNROLL>{}, std::false_type{});
+  switch (count) {
+    case 4: if (UNROLL >= 4) group(std::integral_constant<int, (UNROLL >= 4 ? 4 : 1)>{}, std::true_type{}); break;
+    case 3: if (UNROLL >= 3) group(std::integral_constant<int, (UNROLL >= 3 ? 3 : 1)>{}, std::true_type{}); break;
+    case 2: if (UNROLL >= 2) group(std::integral_constant<int, (UNROLL >= 2 ? 2 : 1)>{}, std::true_type{}); break;
+    case 1: group(std::integral_constant<int, 1>{}, std::true_type{}); break;
     default: break;
   }
-  if (k0 < K) {                                 // the chunk that K cuts (K is a multiple of 8, a chunk is 32 wide)
-    const bool kin = k0 + fk < K;
-    const int ks = kin ? k0 : -fk;              // a load that is not wanted reads the row's first chunk and is dropped
-    uint4 wv = load16(wp + ks);
-    if (!kin) wv = make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      uint4 av = load16(ap[i] + ks);
-      if (!kin) av = make_uint4(0, 0, 0, 0);
-      acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                       __builtin_bit_cast(bf16x8_t, wv), acc[i], 0, 0, 0);
-    }
-  }
+  lds_barrier();
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (SK_COLS == 16 || fr < SK_COLS) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
+    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, ml = e / SK_COLS, m = r0 + ml, c = e % SK_COLS, n = n0 + c;
-    if (e < MT * 16 * SK_COLS && m < M && n < N) {
+    const int e = t + j * NW * 64, ml = e / 16, m = r0 + ml, c = e % 16, n = n0 + c;
+    if (e < AR * 16 && m < M && n < N) {
       float v = red[0][ml][c];
 #pragma unroll
       for (int v2 = 1; v2 < NW; ++v2) v += red[v2][ml][c];
@@ -364,20 +388,42 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   }
 }
 
+template <int NW>
+static int launch_skinny(int mt, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
+                         const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
+  dim3 grid(da_ceil_div(N, 16)), block(NW * 64);
+  // With few columns the row tiles are spread over more workgroups (blockIdx.y), as long as the chip
+  // is not full: each then reads fewer rows of a.  A row's sums do not depend on it.
+  for (int mb = 1; mb < mt; mb *= 2)
+    if ((long)grid.x * da_ceil_div(mt, mb) <= 256) {
+      grid.y = da_ceil_div(mt, mb);
+      mt = mb;
+      break;
+    }
+  DA_REQUIRE(mt >= 1 && mt <= 4, "gemm_bf16: %d row tiles", mt);
+  // steps in flight: 16 to 20 loads of 16 bytes a lane
+  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 4>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 3>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  return 0;
+}
+
 // ---------------------------------------------------------------------------------------------
-// M <= 16.  MFMA 4x4x4: 16 independent 4x4 products of depth 4 a wavefront.  Lane l gives row (a) /
+// M <= 4 and up to 2,048 columns (a decode step of a few requests).  MFMA 4x4x4: 16 independent 4x4
+// products of depth 4 a wavefront.  Lane l gives row (a) /
 // column (b) l % 4 of product l / 4 and 4 consecutive k; it receives column l % 4 of that product,
 // rows 0..3.  The 16 products of a step take 16 consecutive pieces of k of 8 elements (two
 // instructions each), so a lane loads 16 bytes and the 16 lanes of one row of w read 256 consecutive
-// bytes: whole cache lines.  (The 16x16x32 form reads 16 rows x 64 bytes a load, and a compute unit's
-// L1 passes that at a third of the rate.)  A workgroup owns 4 * NG columns; wavefront v of NW takes
+// bytes: whole cache lines without a detour through LDS.  A workgroup owns 4 * NG columns; wavefront v of NW takes
 // the steps v, v+NW, ... of 128 elements of k; the products of a wavefront are summed over its 16
 // lanes-groups at the end (two lane rotations, then LDS) in a fixed order.
 // ---------------------------------------------------------------------------------------------
-template <int MG, int NG, int NW, int UNROLL>
+template <int NG, int NW, int UNROLL>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny4_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                     Epilogue ep, KvScatter kv, int M, int N, int K) {
+  constexpr int MG = 1;                        // row groups of 4 (from 5 rows on gemm_skinny is faster)
   constexpr int ROWS = MG * 4, COLS = NG * 4;
   __shared__ __attribute__((aligned(16))) float red[4 * NW][COLS][ROWS];
   static_assert(NW * 64 >= 4 * ROWS * COLS, "four threads an output element");
@@ -502,38 +548,15 @@ gemm_skinny4_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restr
   }
 }
 
-template <int MG, int NG>
+template <int NG>
 static int launch_skinny4(int nw, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
                           const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
-  static_assert(MG * NG <= 8, "four threads an output element in 16 wavefronts at most");
-  DA_REQUIRE(M <= MG * 4, "gemm_bf16: %d rows for %d groups of 4", M, MG);
+  DA_REQUIRE(M <= 4, "gemm_bf16: %d rows for one group of 4", M);
   const dim3 grid(da_ceil_div(N, NG * 4));
-  constexpr int U = MG + NG <= 4 ? 4 : (MG + NG <= 6 ? 3 : 2);
-  // (4 wavefronts are too few threads for 8 groups: 8 then)
-#define DA_SK4_GO(NWv) hipLaunchKernelGGL((gemm_skinny4_kernel<MG, NG, (NWv < MG * NG ? 8 : NWv), U>), grid, dim3((NWv < MG * NG ? 8 : NWv) * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K)
-  if (nw > 8) DA_SK4_GO(16);
-  else if (nw > 4) DA_SK4_GO(8);
-  else DA_SK4_GO(4);
-#undef DA_SK4_GO
+  if (nw == 16) hipLaunchKernelGGL((gemm_skinny4_kernel<NG, 16, 4>), grid, dim3(1024), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (nw == 8) hipLaunchKernelGGL((gemm_skinny4_kernel<NG, 8, 4>), grid, dim3(512), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny4_kernel<NG, 4, 4>), grid, dim3(256), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
   return 0;
-}
-
-template <int NW, int COLS>
-static void launch_skinny(int mt, dim3 grid, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
-                          const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
-  // With few columns the row tiles are spread over more workgroups (blockIdx.y), as long as the chip
-  // is not full: each then reads fewer rows of a.  A row's sums do not depend on it.
-  for (int mb = 1; mb < mt; mb *= 2)
-    if ((long)grid.x * da_ceil_div(mt, mb) <= 256) {
-      grid.y = da_ceil_div(mt, mb);
-      mt = mb;
-      break;
-    }
-  // few rows leave registers for more chunks in flight
-  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 8, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 4, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2, COLS>), grid, dim3(NW * 64), 0, s, A, lda, W, ldw, ep, kv, M, N, K);
 }
 
 extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
@@ -557,33 +580,19 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
-  if (M <= 16 && N <= 2048 && (M <= 8 || K >= 2048)) {
-    // Measured: the 4x4x4 form wins where few workgroups pull on memory (up to 2,048 columns; by 25 to 40 %
-    // with K from 2,048 on).  With more columns both forms stream alike and the other one's sums are cheaper;
-    // beyond 8 rows the loads of a outweigh it unless K is large.
-    const int mg = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
-    const int ng = N <= 1024 ? 1 : 2;
+  if (M <= 4 && N <= 2048) {
+    // Measured: up to 4 rows and 2,048 columns the 4x4x4 form is ahead, by 20 to 25 % with K from 2,048 on.
     const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // by K alone, so a row's sums keep their order
-#define DA_SK4(MG, NG) launch_skinny4<MG, NG>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)
-    int rc;
-    if (ng == 1) rc = mg == 1 ? DA_SK4(1, 1) : (mg == 2 ? DA_SK4(2, 1) : DA_SK4(4, 1));
-    else rc = mg == 1 ? DA_SK4(1, 2) : (mg == 2 ? DA_SK4(2, 2) : DA_SK4(4, 2));
-    if (rc) return rc;
-#undef DA_SK4
+    if (N <= 1024 ? launch_skinny4<1>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)
+                  : launch_skinny4<2>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)) return 1;
   } else if (M <= 64) {
+    // The number of wavefronts that split K depends on K and N alone, so a row's sums keep their order:
+    // 4 where the workgroups are many (a vocabulary: several then share a compute unit), else 8, or 12 for a long K.
     const int mt = da_ceil_div(M, 16);
-    // 8 columns a workgroup where 16 would leave most compute units without one (one row tile only)
-    const int cols = (mt == 1 && da_ceil_div(N, 16) <= 64) ? 8 : 16;
-    dim3 grid(da_ceil_div(N, cols));
-    // the number of wavefronts that split K depends on K alone, so a row's sums keep their order
-    const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // measured: larger blocks cost more than they hide
-    if (cols == 8) {
-      if (nw == 16) launch_skinny<16, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-      else if (nw == 8) launch_skinny<8, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-      else launch_skinny<4, 8>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    } else if (nw == 16) launch_skinny<16, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else if (nw == 8) launch_skinny<8, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
-    else launch_skinny<4, 16>(mt, grid, s, A, lda, W, ldw, ep, kv, M, N, K);
+    const int nw = da_ceil_div(N, 16) > 1024 ? 4 : (K >= 2048 ? 12 : 8);
+    if (nw == 4 ? launch_skinny<4>(mt, s, A, lda, W, ldw, ep, kv, M, N, K)
+                : (nw == 8 ? launch_skinny<8>(mt, s, A, lda, W, ldw, ep, kv, M, N, K)
+                           : launch_skinny<12>(mt, s, A, lda, W, ldw, ep, kv, M, N, K))) return 1;
   } else {
     // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
     // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so

@@ -102,8 +102,9 @@ def test_gemm_plain_32bit(ops, M, N, K):
 @pytest.mark.parametrize("M", [1, 3, 5, 8, 12, 16, 17, 40, 64, 65, 128, 200, 513])
 @pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24), (300, 2056), (1030, 1160)])
 def test_gemm_matrix_cores(ops, M, N, K):
-    """Every kernel form behind ``linear_mfma`` (few rows and few columns: 4x4x4 products with 1, 2 or 4
-    row groups, 4 to 16 wavefronts, a last step that K cuts; few rows: 16x16x32; else block tiles)."""
+    """Every kernel form behind ``linear_mfma`` (up to 4 rows and 2,048 columns: 4x4x4 products, 4 to 16
+    wavefronts; up to 64 rows: 16x16x32 products fed through LDS, 1 to 4 row tiles, 8 or 12 wavefronts;
+    else block tiles), each with a last step that K cuts."""
     g = torch.Generator().manual_seed(M * 7 + N)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
                                (None, True, True, torch.float32), (None, False, False, torch.float32),
@@ -115,7 +116,7 @@ def test_gemm_matrix_cores(ops, M, N, K):
 
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """A row's result is the same, bit for bit, whatever other rows share the call, as long as the call
-    takes the same kernel form (block tiles; 16x16x32 products for 9 to 64 rows; 4x4x4 products up to 8
+    takes the same kernel form (block tiles; 16x16x32 products up to 64 rows; 4x4x4 products up to 4
     rows and 2,048 columns); between forms it differs by the rounding of 32-bit sums at most."""
     g = torch.Generator().manual_seed(3)
     K, N = 768, 300
@@ -131,7 +132,8 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     assert torch.equal(rows(60, 150), full[60:150])                 # block tiles
     small = rows(0, 64)
     assert torch.equal(rows(3, 23)[7], small[10])                   # 16x16x32: 20 rows, 64 rows
-    assert torch.equal(rows(10, 11)[0], rows(4, 12)[6])             # 4x4x4: 1 row, 8 rows
+    assert torch.equal(rows(4, 12)[6], small[10])                   # ... 8 rows
+    assert torch.equal(rows(10, 11)[0], rows(8, 12)[2])             # 4x4x4: 1 row, 4 rows
     assert torch.equal(rows(10, 13)[0], rows(10, 11)[0])            # ... 3 rows
     exact = a[10].double() @ w.double().t()
     scale = exact.abs().max().item()
