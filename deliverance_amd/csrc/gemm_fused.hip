@@ -180,96 +180,86 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 }
 
 // ---------------------------------------------------------------------------------------------
-// The same for up to 16 rows and K <= CH * NW * 32, with every load asked for at the start: the
-// wavefront's CH chunks of w, the matching pieces of the rows, of the gain and of the bias, and the
-// rows for the statistics.  The kernel then costs one memory round trip, two reductions, the
-// products and the merge of the wavefronts.  Wavefront v takes the chunks v, v + NW, ...; the sum
-// over k runs in that order, whatever M is.
+// One row tile (M <= 16), K <= 2048, parameters of one dtype: every load in whole cache lines.
+// Wavefront v of 8 reads rows v and v + 8 whole (RV float4 a lane), with the gain and bias at the
+// same places, computes their statistics, and writes the normalised rows as bfloat16 into LDS,
+// zeros past K.  The steps of w (64 elements of k, 8 rows x 128 bytes a load; wavefront v takes the
+// steps v, v + 8, ...) are asked for before anything else is computed and parked in the wavefront's
+// own piece of LDS; the fragments of both operands are read from LDS.  Steps past K read step 0 and
+// meet zeros.  The sum over k runs in the order of the steps, whatever M is.
 // ---------------------------------------------------------------------------------------------
-// Parameters (gain, bias of the norm, bias of the product) are loaded as raw bits and converted
-// where they are used: a conversion right after its load would wait for it, and for every load
-// asked for before it.  PBF16: the three are bfloat16 (else 32-bit).
-template <bool PBF16>
-struct Raw8 {                       // 8 consecutive parameter values as loaded
-  uint4 a, b;                       // bfloat16: a only
-  __device__ __forceinline__ void load(const void* p, int i) {
-    if (PBF16) a = *(const uint4*)((const bf16_t*)p + i);
-    else { a = *(const uint4*)((const float*)p + i); b = *(const uint4*)((const float*)p + i + 4); }
-  }
-  __device__ __forceinline__ void get(float* o) const {
-    if (PBF16) {
-      const uint32_t v[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) { o[2 * e] = __uint_as_float(v[e] << 16); o[2 * e + 1] = __uint_as_float(v[e] & 0xffff0000u); }
-    } else {
-      const uint32_t v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = __uint_as_float(v[e]);
-    }
-  }
-};
-
-// (a decode step's products have at most about one workgroup per compute unit, so registers are not held down)
-template <int NW, int CH, bool PBF16>
-__global__ void __launch_bounds__(NW * 64, 2)
+#define FL_LD (64 + 8)       // padded row of a parked step of w, elements
+template <int RV, bool PBF16>
+__global__ void __launch_bounds__(512)
 gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
-                    int M, int N, int K) {
-  constexpr int RV = (CH * NW * 32 / 4 + 63) / 64;          // float4 per lane when a row is held in registers
+                   int M, int N, int K) {
+  constexpr int NW = 8, KMAX = RV * 256, ALD = KMAX + 8;      // ALD: padded row of a in LDS, elements
+  constexpr int SW = (RV * 4 + NW - 1) / NW;                   // steps a wavefront
+  __shared__ __attribute__((aligned(16))) bf16_t a_lds[16][ALD];
+  __shared__ __attribute__((aligned(16))) bf16_t stage[NW][16 * FL_LD];
   __shared__ float red[NW][16][FZ_COLS + 1];
-  __shared__ float s_mean[16], s_rstd[16];
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int n0 = blockIdx.x * FZ_COLS;
-  const int fr = lane % 16, fk = (lane / 16) * 8;
-  const bool arow_ok = fr < M;
-  const int arow = arow_ok ? fr : 0;
-  const float* xp = ln.x + (size_t)(ln.rows ? ln.rows[arow] : arow) * K + fk;
-  const bf16_t* wp = w + (size_t)(n0 + fr < N ? n0 + fr : N - 1) * ldw + fk;    // columns past N are never stored
+  const int fr = lane % 16, fk = (lane / 16) * 8;    // a fragment: row fr of 16, k-group lane / 16
+  const int lr = lane / 8, lc = (lane % 8) * 8;      // a load of w: row lr of 8, 16-byte piece lane % 8
 
-  // Loads come back in the order they were asked for, so they are asked for in the order of their
-  // use: the rows for the statistics (wavefront v takes rows v and v + NW), the pieces of the rows,
-  // of the gain and of the bias for the products, what the epilogue needs, and last the chunks of w,
-  // which come from furthest away.  Nothing is computed before all are on their way.
+  // ---- all loads first, in the order of their use
+  // (rows from M on are neither read nor normalised: what they give is never stored; the row number
+  // is made a scalar so that the branch around their loads is one for the whole wavefront)
+  const int row0 = __builtin_amdgcn_readfirstlane(wave);
   float4 sv[2][RV];
+  uint4 gq[RV], bq[RV];                              // gain and bias at this lane's places (bfloat16: .x .y only)
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int m = wave + j * NW, ms = m < M ? m : 0;
-    const float* xr = ln.x + (size_t)(ln.rows ? ln.rows[ms] : ms) * K;
+    const int m = row0 + j * NW;
+    if (m < M) {
+      const float* xr = ln.x + (size_t)(ln.rows ? ln.rows[m] : m) * K;
 #pragma unroll
-    for (int i = 0; i < RV; ++i) {
-      const int c = (lane + i * 64) * 4;
-      sv[j][i] = *(const float4*)(xr + (c < K ? c : 0));
+      for (int i = 0; i < RV; ++i) {
+        const int c = (lane + i * 64) * 4;
+        sv[j][i] = *(const float4*)(xr + (c < K ? c : 0));
+      }
     }
   }
-  float4 xa[CH][2];
-  Raw8<PBF16> gr[CH], br[CH];
-  int ks[CH];
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    const int k = (wave + c * NW) * 32;
-    ks[c] = (k + fk < K) ? k : -fk;               // past K: the row's first piece, met by zeros in a
-    xa[c][0] = *(const float4*)(xp + ks[c]);
-    xa[c][1] = *(const float4*)(xp + ks[c] + 4);
-    gr[c].load(ln.g, ks[c] + fk);
-    if (ln.b) br[c].load(ln.b, ks[c] + fk);
+  for (int i = 0; i < RV; ++i) {
+    const int c = (lane + i * 64) * 4, cs = c < K ? c : 0;
+    if (PBF16) {
+      const uint2 g2 = *(const uint2*)((const bf16_t*)ln.g + cs);
+      gq[i] = make_uint4(g2.x, g2.y, 0, 0);
+      const uint2 b2 = *(const uint2*)((const bf16_t*)(ln.b ? ln.b : ln.g) + cs);
+      bq[i] = make_uint4(b2.x, b2.y, 0, 0);
+    } else {
+      gq[i] = *(const uint4*)((const float*)ln.g + cs);
+      bq[i] = *(const uint4*)((const float*)(ln.b ? ln.b : ln.g) + cs);
+    }
   }
   // this thread's output element (16 x 16 of them), with what its epilogue needs
   const int em = t / FZ_COLS, ec = t % FZ_COLS, en = n0 + ec;
   const bool e_ok = t < 16 * FZ_COLS && em < M && en < N;
   const int ebn = e_ok ? en : 0;
-  // (without a bias some valid place is read and dropped: a load inside a branch is waited for there)
   const void* e_bsrc = ep.bias ? ep.bias : (const void*)w;
   const int e_bidx = ep.bias ? ebn : 0;
   const uint32_t e_bias_raw = PBF16 ? (uint32_t)((const bf16_t*)e_bsrc)[e_bidx] : ((const uint32_t*)e_bsrc)[e_bidx];
   const int e_slot = kv.cache ? kv.slot_map[e_ok ? em : 0] : -1;
-  uint4 wv[CH];
+  uint4 wv[SW][2];
 #pragma unroll
-  for (int c = 0; c < CH; ++c) wv[c] = load16(wp + ks[c]);
-  __builtin_amdgcn_sched_barrier(0);              // the loads stay in this order, ahead of the arithmetic
+  for (int u = 0; u < SW; ++u) {
+    const int k0 = (wave + u * NW) * 64;
+    const int kk = k0 + lc < K ? k0 + lc : 0;        // past K: the row's first piece
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int n = n0 + i * 8 + lr;
+      wv[u][i] = load16(w + (size_t)(n < N ? n : 0) * ldw + kk);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);                 // the loads stay in this order, ahead of the arithmetic
 
-  // ---- statistics
+  // ---- statistics and the normalised rows
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int m = wave + j * NW;
+    const int m = row0 + j * NW;
+    if (m >= M) continue;
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < RV; ++i) {
@@ -285,31 +275,56 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
       q += (c < K ? 1.f : 0.f) * ((d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3));
     }
     const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)K + ln.eps);
-    if (lane == 0 && m < M) { s_mean[m] = mean; s_rstd[m] = rstd; }
+#pragma unroll
+    for (int i = 0; i < RV; ++i) {
+      const int c = (lane + i * 64) * 4;
+      float g4[4], b4[4];
+      if (PBF16) {
+        g4[0] = __uint_as_float(gq[i].x << 16); g4[1] = __uint_as_float(gq[i].x & 0xffff0000u);
+        g4[2] = __uint_as_float(gq[i].y << 16); g4[3] = __uint_as_float(gq[i].y & 0xffff0000u);
+        b4[0] = __uint_as_float(bq[i].x << 16); b4[1] = __uint_as_float(bq[i].x & 0xffff0000u);
+        b4[2] = __uint_as_float(bq[i].y << 16); b4[3] = __uint_as_float(bq[i].y & 0xffff0000u);
+      } else {
+        g4[0] = __uint_as_float(gq[i].x); g4[1] = __uint_as_float(gq[i].y); g4[2] = __uint_as_float(gq[i].z); g4[3] = __uint_as_float(gq[i].w);
+        b4[0] = __uint_as_float(bq[i].x); b4[1] = __uint_as_float(bq[i].y); b4[2] = __uint_as_float(bq[i].z); b4[3] = __uint_as_float(bq[i].w);
+      }
+      const float xs[4] = {sv[j][i].x, sv[j][i].y, sv[j][i].z, sv[j][i].w};
+      float y[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        y[e] = (xs[e] - mean) * rstd * g4[e];
+        if (ln.b) y[e] += b4[e];
+      }
+      uint2 pk = make_uint2((uint32_t)f32_to_bf16(y[0]) | ((uint32_t)f32_to_bf16(y[1]) << 16),
+                            (uint32_t)f32_to_bf16(y[2]) | ((uint32_t)f32_to_bf16(y[3]) << 16));
+      if (c >= K) pk = make_uint2(0, 0);
+      *(uint2*)&a_lds[m][c] = pk;
+    }
   }
   lds_barrier();
-  const float mean = s_mean[arow], rstd = s_rstd[arow];
 
+  // ---- products: a step of w is parked, then both operands' fragments come out of LDS
+  bf16_t* mine = stage[wave];
   floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    const bool kin = (wave + c * NW) * 32 + fk < K;
-    const float xs[8] = {xa[c][0].x, xa[c][0].y, xa[c][0].z, xa[c][0].w, xa[c][1].x, xa[c][1].y, xa[c][1].z, xa[c][1].w};
-    float gg[8], bb[8];
-    gr[c].get(gg);
-    if (ln.b) br[c].get(bb);
-    uint32_t pk[4];
+  for (int u = 0; u < SW; ++u) {
+    const int k0 = (wave + u * NW) * 64;             // < KMAX: the rows of a are zero from K on
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float y0 = (xs[2 * e] - mean) * rstd * gg[2 * e];
-      float y1 = (xs[2 * e + 1] - mean) * rstd * gg[2 * e + 1];
-      if (ln.b) { y0 += bb[2 * e]; y1 += bb[2 * e + 1]; }
-      pk[e] = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
+    for (int i = 0; i < 2; ++i) *(uint4*)&mine[(i * 8 + lr) * FL_LD + lc] = wv[u][i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (SW * NW * 64 <= KMAX || k0 < KMAX) {
+#pragma unroll
+      for (int c = 0; c < 64; c += 32) {
+        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[fr * FL_LD + c + fk]);
+        const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&a_lds[fr][k0 + c + fk]);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc, 0, 0, 0);
+      }
     }
-    uint4 av = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-    if (!(kin && arow_ok)) av = make_uint4(0, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, wv[c]),
-                                                  acc, 0, 0, 0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][4 * (lane / 16) + r][fr] = acc[r];
@@ -353,21 +368,24 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
   dim3 grid(da_ceil_div(N, FZ_COLS));
   const int mt = da_ceil_div(M, 16);
   hipStream_t s = (hipStream_t)stream;
-  // the kernel with all loads up front takes one row tile, K up to 1024, and parameters of one dtype
+  // the kernel with whole-line loads takes one row tile, K up to 2048, and parameters of one dtype
   const int pdt = g_dtype;
   const bool same = (!b || b_dtype == pdt) && (!bias || bias_dtype == pdt) && (pdt == DA_BF16 || pdt == DA_F32);
-#define LAUNCH_ROWS(CH)                                                                                           \
+#define LAUNCH_LDS(RV)                                                                                            \
   do {                                                                                                            \
     if (pdt == DA_BF16)                                                                                           \
-      hipLaunchKernelGGL((gemm_ln_rows_kernel<8, CH, true>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, true>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
     else                                                                                                          \
-      hipLaunchKernelGGL((gemm_ln_rows_kernel<8, CH, false>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, false>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
   } while (0)
-  if (mt == 1 && same && K <= 2 * 8 * 32) LAUNCH_ROWS(2);
-  else if (mt == 1 && same && K <= 3 * 8 * 32) LAUNCH_ROWS(3);
-  else if (mt == 1 && same && K <= 4 * 8 * 32) LAUNCH_ROWS(4);
-#undef LAUNCH_ROWS
-  else
+  if (mt == 1 && same && K <= 2048) {
+    if (K <= 256) LAUNCH_LDS(1);
+    else if (K <= 512) LAUNCH_LDS(2);
+    else if (K <= 768) LAUNCH_LDS(3);
+    else if (K <= 1024) LAUNCH_LDS(4);
+    else if (K <= 1536) LAUNCH_LDS(6);
+    else LAUNCH_LDS(8);
+  } else
     // 8 wavefronts, two chunks in flight each: 125 registers, so two workgroups share a compute unit
     // (deeper unrolling needs 168 and halves that; 16 wavefronts spill)
     launch_fused<8, 2>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);

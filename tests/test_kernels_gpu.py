@@ -420,14 +420,17 @@ def test_xtc_and_logprobs(ops):
 
 # ----------------------------------------------------------------------------- fused norm + product
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 2304, 768), (17, 1000, 96), (32, 200, 1600), (5, 50257, 768),
-                                   (16, 520, 1024), (12, 72, 1000), (9, 40, 520)])
+                                   (16, 520, 1024), (12, 72, 1000), (9, 40, 520), (3, 1000, 1600), (16, 300, 2048),
+                                   (5, 64, 1304), (2, 48, 8), (11, 200, 1992)])
 @pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_product(ops, M, N, K, pdtype):
     g = torch.Generator().manual_seed(M + N)
     x = (torch.randn(M + 3, K, generator=g) * 2 + 1).to(DEV)
     gw, gb = torch.randn(K, generator=g).to(pdtype).to(DEV), torch.randn(K, generator=g).to(pdtype).to(DEV)
     w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
-    bias = bf(torch.randn(N, generator=g)).to(DEV)
+    # the product's bias in the norm's dtype (the kernels for parameters of one dtype) or, with 32-bit norm
+    # parameters and an even M, in bfloat16 (the general kernel)
+    bias = bf(torch.randn(N, generator=g)).to(pdtype if M % 2 else torch.bfloat16).to(DEV)
     rows = torch.tensor([(i * 7) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
     a = F.layer_norm(x.double(), (K,), gw.double(), gb.double(), 1e-5)[rows.long()].to(torch.bfloat16).double()
     for act, od in ((None, torch.float32), ("gelu_new", torch.bfloat16)):
