@@ -253,44 +253,48 @@ static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
 // of the rate, and that rate, not the memory's, bounds a workgroup.)
 // ---------------------------------------------------------------------------------------------
 #define SK_LD (64 + 8)       // padded row of a step in LDS, elements (144 bytes)
-template <int MT, int NW, int UNROLL>
+// AL: loads of 8 rows that cover the workgroup's rows of a (1: up to 8 rows; else two a row tile);
+// COLS: 16 output columns a workgroup, or 8 (the fragment of w then holds them twice and half of the
+// result is dropped: with few columns twice the workgroups pull on memory).
+template <int AL, int COLS, int NW, int UNROLL>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                       Epilogue ep, KvScatter kv, int M, int N, int K) {
-  constexpr int AR = MT * 16, TR = AR + 16;          // rows of a; rows of a step: a's, then w's 16
-  constexpr int AL = MT * 2;                         // loads of 8 rows that cover a
+                   Epilogue ep, KvScatter kv, int M, int N, int K) {
+  constexpr int MT = (AL + 1) / 2, WL = COLS / 8;    // row tiles of 16; loads of 8 rows that cover w's columns
+  constexpr int AR = MT * 16, TR = AR + COLS;        // rows of a; rows of a step: a's, then w's
+  static_assert(COLS == 8 || COLS == 16, "8 or 16 columns a workgroup");
   // the wavefronts' partial sums take the place of the parked steps once all products are done
-  constexpr int STAGE_BYTES = NW * TR * SK_LD * 2, RED_BYTES = NW * AR * 17 * 4;
+  constexpr int STAGE_BYTES = NW * TR * SK_LD * 2, RED_BYTES = NW * AR * (COLS + 1) * 4;
   __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES];
   bf16_t (*stage)[TR * SK_LD] = (bf16_t (*)[TR * SK_LD])smem;
-  float (*red)[AR][17] = (float (*)[AR][17])smem;
+  float (*red)[AR][COLS + 1] = (float (*)[AR][COLS + 1])smem;
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * COLS;
   const int r0 = blockIdx.y * AR;                    // the workgroup's first row
   const int lr = lane / 8, lc = (lane % 8) * 8;      // a load: row lr of 8, 16-byte piece lane % 8
   const int fr = lane % 16, fk = (lane / 16) * 8;    // a fragment: row fr of 16, k-group lane / 16
   const bf16_t* pa[AL];
-  const bf16_t* pw[2];
+  const bf16_t* pw[WL];
 #pragma unroll
   for (int i = 0; i < AL; ++i) {
     const int m = r0 + i * 8 + lr;
     pa[i] = a + (size_t)(m < M ? m : 0) * lda + lc;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < WL; ++i) {
     const int n = n0 + i * 8 + lr;
     pw[i] = w + (size_t)(n < N ? n : 0) * ldw + lc;
   }
   // what the epilogue needs is asked for first, as raw bits from places that always exist
-  constexpr int EPT = (AR * 16 + NW * 64 - 1) / (NW * 64);
+  constexpr int EPT = (AR * COLS + NW * 64 - 1) / (NW * 64);
   uint32_t e_braw[EPT];
   float e_old[EPT];
   int e_slot[EPT];
   const bool bias_bf16 = ep.bias_dtype == DA_BF16;
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, m = r0 + e / 16, n = n0 + e % 16;
-    const bool ok = e < AR * 16 && m < M && n < N;
+    const int e = t + j * NW * 64, m = r0 + e / COLS, n = n0 + e % COLS;
+    const bool ok = e < AR * COLS && m < M && n < N;
     const void* bsrc = (ok && ep.bias) ? ep.bias : (const void*)w;
     const int bidx = (ok && ep.bias) ? n : 0;
     e_braw[j] = bias_bf16 ? (uint32_t)((const bf16_t*)bsrc)[bidx] : ((const uint32_t*)bsrc)[bidx];
@@ -301,6 +305,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   bf16_t* mine = stage[wave];
+  // (With AL == 1 the rows 8..15 of the tile are never parked: whatever LDS holds there gives rows of
+  // the result that are never stored.)
   // The wavefront's steps (v, v+NW, ...) go two at a time: all loads of both first, then each is
   // parked in LDS and multiplied.  The very last step may be the one that K cuts: lanes past K read
   // the row's first piece instead and park zeros.
@@ -310,7 +316,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
   auto group = [&](auto gc, auto lastc) {
     constexpr int G = decltype(gc)::value;
     constexpr bool LAST = decltype(lastc)::value;
-    uint4 av[G][AL], wv[G][2];
+    uint4 av[G][AL], wv[G][WL];
     bool kin = true;
 #pragma unroll
     for (int u = 0; u < G; ++u) {
@@ -322,27 +328,27 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 #pragma unroll
       for (int i = 0; i < AL; ++i) av[u][i] = load16(pa[i] + kk);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) wv[u][i] = load16(pw[i] + kk);
+      for (int i = 0; i < WL; ++i) wv[u][i] = load16(pw[i] + kk);
     }
 #pragma unroll
     for (int u = 0; u < G; ++u) {
 #pragma unroll
       for (int i = 0; i < AL; ++i) *(uint4*)&mine[(i * 8 + lr) * SK_LD + lc] = av[u][i];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = wv[u][i];
+      for (int i = 0; i < WL; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = wv[u][i];
       if (LAST && u == G - 1 && !kin) {        // past K: zeros over what the lane just parked
         const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < AL; ++i) *(uint4*)&mine[(i * 8 + lr) * SK_LD + lc] = zero;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = zero;
+        for (int i = 0; i < WL; ++i) *(uint4*)&mine[(AR + i * 8 + lr) * SK_LD + lc] = zero;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 #pragma unroll
       for (int c = 0; c < 64; c += 32) {
-        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[(AR + fr) * SK_LD + c + fk]);
+        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[(AR + fr % COLS) * SK_LD + c + fk]);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
           const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[(i * 16 + fr) * SK_LD + c + fk]);
@@ -368,12 +374,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
+    for (int r = 0; r < 4; ++r)
+      if (COLS == 16 || fr < COLS) red[wave][i * 16 + 4 * (lane / 16) + r][fr] = acc[i][r];
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = t + j * NW * 64, ml = e / 16, m = r0 + ml, c = e % 16, n = n0 + c;
-    if (e < AR * 16 && m < M && n < N) {
+    const int e = t + j * NW * 64, ml = e / COLS, m = r0 + ml, c = e % COLS, n = n0 + c;
+    if (e < AR * COLS && m < M && n < N) {
       float v = red[0][ml][c];
 #pragma unroll
       for (int v2 = 1; v2 < NW; ++v2) v += red[v2][ml][c];
@@ -389,9 +396,18 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 }
 
 template <int NW>
-static int launch_skinny(int mt, hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
+static int launch_skinny(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw,
                          const Epilogue& ep, const KvScatter& kv, int M, int N, int K) {
-  dim3 grid(da_ceil_div(N, 16)), block(NW * 64);
+  const dim3 block(NW * 64);
+  int mt = da_ceil_div(M, 16);
+#define DA_SK_GO(AL, COLS, U) hipLaunchKernelGGL((gemm_skinny_kernel<AL, COLS, NW, U>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K)
+  if (mt == 1 && NW != 4 && da_ceil_div(N, 16) < 128) {
+    // few columns and one row tile: 8 columns a workgroup
+    const dim3 grid(da_ceil_div(N, 8));
+    if (M <= 8) DA_SK_GO(1, 8, 4); else DA_SK_GO(2, 8, 4);
+    return 0;
+  }
+  dim3 grid(da_ceil_div(N, 16));
   // With few columns the row tiles are spread over more workgroups (blockIdx.y), as long as the chip
   // is not full: each then reads fewer rows of a.  A row's sums do not depend on it.
   for (int mb = 1; mb < mt; mb *= 2)
@@ -402,10 +418,12 @@ static int launch_skinny(int mt, hipStream_t s, const bf16_t* A, int lda, const 
     }
   DA_REQUIRE(mt >= 1 && mt <= 4, "gemm_bf16: %d row tiles", mt);
   // steps in flight: 16 to 20 loads of 16 bytes a lane
-  if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, NW, 4>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, NW, 3>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, NW, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<4, NW, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K);
+  if (mt == 1 && M <= 8) DA_SK_GO(1, 16, 4);
+  else if (mt == 1) DA_SK_GO(2, 16, 4);
+  else if (mt == 2) DA_SK_GO(4, 16, 3);
+  else if (mt == 3) DA_SK_GO(6, 16, 2);
+  else DA_SK_GO(8, 16, 2);
+#undef DA_SK_GO
   return 0;
 }
 
@@ -585,14 +603,13 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     const int nw = K >= 2048 ? 16 : (K >= 1024 ? 8 : 4);   // by K alone, so a row's sums keep their order
     if (N <= 1024 ? launch_skinny4<1>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)
                   : launch_skinny4<2>(nw, s, A, lda, W, ldw, ep, kv, M, N, K)) return 1;
-  } else if (M <= 64) {
+  } else if (M <= 32 || (M <= 64 && N <= 8192)) {     // (a vocabulary with more than 32 rows: block tiles reuse the rows of a)
     // The number of wavefronts that split K depends on K and N alone, so a row's sums keep their order:
     // 4 where the workgroups are many (a vocabulary: several then share a compute unit), else 8, or 12 for a long K.
-    const int mt = da_ceil_div(M, 16);
     const int nw = da_ceil_div(N, 16) > 1024 ? 4 : (K >= 2048 ? 12 : 8);
-    if (nw == 4 ? launch_skinny<4>(mt, s, A, lda, W, ldw, ep, kv, M, N, K)
-                : (nw == 8 ? launch_skinny<8>(mt, s, A, lda, W, ldw, ep, kv, M, N, K)
-                           : launch_skinny<12>(mt, s, A, lda, W, ldw, ep, kv, M, N, K))) return 1;
+    if (nw == 4 ? launch_skinny<4>(s, A, lda, W, ldw, ep, kv, M, N, K)
+                : (nw == 8 ? launch_skinny<8>(s, A, lda, W, ldw, ep, kv, M, N, K)
+                           : launch_skinny<12>(s, A, lda, W, ldw, ep, kv, M, N, K))) return 1;
   } else {
     // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
     // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so
