@@ -10,7 +10,7 @@ to each other for the attention kernels.  All slots of a group live in one alloc
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import Dict, List
 
 import torch
 

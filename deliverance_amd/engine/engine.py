@@ -23,7 +23,6 @@ import torch
 from ..config.engine_config import EngineConfig
 from ..kernels import ops
 from ..models.causal_lm import CausalLM, load_model
-from ..parts.base import KVNeed
 from ..profiler import InferenceProfiler
 from ..sampling.params import GeneratorParameters
 from ..sampling.sampler import RECORD_WORDS, device_record

@@ -13,7 +13,7 @@ from __future__ import annotations
 
 import math
 import struct
-from typing import List, Optional
+from typing import Optional
 
 from .params import GeneratorParameters
 
