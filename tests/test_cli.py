@@ -33,3 +33,20 @@ def test_help_names_the_reference_options():
         assert opt in p.stdout
     p = run("generate", "--model", "/nonexistent")
     assert p.returncode != 0
+
+
+def test_bench_measures_one_gpu_only():
+    """With more than one GPU asked for, bench.py says so in one line and exits with 2."""
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 2
+    assert len(p.stdout.strip().splitlines()) == 1 and "--gpus 2" in p.stdout
+
+
+def test_trace_run_without_a_gpu_says_so(tmp_path):
+    """The replay program drives the GPU engine only: without a GPU it ends with a message, not a traceback."""
+    import torch
+    if torch.cuda.is_available():
+        return
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(tmp_path), "--dtype", "float32",
+                        "--out", str(tmp_path / "o"), "--max-tokens", "64"], input="", capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "no GPU is visible" in p.stderr and "Traceback" not in p.stderr
