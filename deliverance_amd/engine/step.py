@@ -37,12 +37,128 @@ class StepError(ValueError):
     pass
 
 
+class StepPacker:
+    """The host side of a step: where each array of the step lies in its one buffer of integers,
+    and the values that go there.  It reads the cache manager only, so it runs without a GPU."""
+
+    def __init__(self, manager, n_groups: int, page_size: int):
+        self.manager = manager
+        self.n_groups = n_groups
+        self.page_size = page_size
+
+    def layout(self, entries, order, pad_to, max_blocks, extra):
+        """Where each array of the step lies in its one buffer of integers: tokens, where a token
+        comes from, positions, sequence ids, row starts, lengths, state slots, wanted rows, then
+        per cache group the cache row of every token and the block tables, then ``extra``.  With
+        ``pad_to`` the step is filled up with empty one-token sequences (length 0, no cache row),
+        so that its shape is fixed."""
+        mgr = self.manager
+        S_real = len(entries)
+        n_pad = 0 if pad_to is None else pad_to - S_real
+        N = sum(len(e.tokens) for e in entries) + n_pad
+        S = S_real + n_pad
+        R = sum(len(e.want) for e in entries) + n_pad
+        G = self.n_groups
+        if max_blocks is None:
+            max_blocks = max(1, max(len(mgr.table(e.rid, g)) for e in entries for g in range(G))) if G else 1
+        n_extra = 0 if not extra else len(extra) + RECORD_WORDS * n_pad
+        offs = {}
+        o = 0
+        for name, n in (("tokens", N), ("token_src", N), ("positions", N), ("seq_of", N), ("q_start", S + 1),
+                        ("seq_lens", S), ("state_slots", S), ("want", R)):
+            offs[name] = (o, n)
+            o += n
+        for g in range(G):
+            offs[f"slot_map{g}"] = (o, N)
+            offs[f"block_table{g}"] = (o + N, S * max_blocks)
+            o += N + S * max_blocks
+        if n_extra:
+            offs["extra"] = (o, n_extra)
+            o += n_extra
+        meta = dict(N=N, S=S, R=R, G=G, max_blocks=max_blocks, n_pad=n_pad,
+                    n_decode=sum(1 for e in entries if len(e.tokens) == 1) + n_pad)
+        return offs, meta, o
+
+    def fill(self, buf, offs, meta, entries, order, starts, extra):
+        """Write the step's integers into ``buf`` (a numpy view of pinned memory).  Long portions
+        are written as arrays, single tokens as scalars."""
+        mgr = self.manager
+        ps = self.page_size
+
+        def view(name):
+            a, n = offs[name]
+            return buf[a:a + n]
+        tok, src, pos, seq = view("tokens"), view("token_src"), view("positions"), view("seq_of")
+        q_start_v, seq_lens_v, state_v, want_v = view("q_start"), view("seq_lens"), view("state_slots"), view("want")
+        G, mb, n_pad = meta["G"], meta["max_blocks"], meta["n_pad"]
+        sms = [view(f"slot_map{g}") for g in range(G)]
+        bts = [view(f"block_table{g}") for g in range(G)]
+        for bt in bts:
+            bt[:] = -1
+        q_start, seq_lens, state_slots = [0], [], []
+        row0 = {}
+        row = 0
+        for s, i in enumerate(order):
+            e = entries[i]
+            n = len(e.tokens)
+            st = starts[e.rid]
+            row0[i] = row
+            if n == 1:
+                tok[row] = e.tokens[0]
+                src[row] = -1 if e.from_sampled is None else e.from_sampled
+                pos[row] = st
+                seq[row] = s
+            else:
+                tok[row:row + n] = e.tokens
+                src[row:row + n] = -1
+                pos[row:row + n] = np.arange(st, st + n, dtype=np.int32)
+                seq[row:row + n] = s
+            for g in range(G):
+                t = mgr.table(e.rid, g)
+                if n == 1:
+                    page = t[st // ps]
+                    if page < 0:
+                        raise StepError(f"position {st} of {e.rid!r} lies in a page that was given back")
+                    sms[g][row] = page * ps + st % ps
+                else:
+                    sms[g][row:row + n] = mgr.slots_for(e.rid, g, st, n)
+                bts[g][s * mb:s * mb + len(t)] = t
+            row += n
+            q_start.append(row)
+            seq_lens.append(st + n)
+            state_slots.append(mgr.state_slot(e.rid))
+        S_real = len(entries)
+        r = 0
+        for i, e in enumerate(entries):
+            for w in e.want:
+                want_v[r] = row0[i] + int(w)
+                r += 1
+        for k in range(n_pad):          # empty one-token sequences
+            tok[row] = 0; src[row] = -1; pos[row] = 0; seq[row] = S_real + k
+            for g in range(G):
+                sms[g][row] = -1
+            want_v[r] = row
+            r += 1
+            row += 1
+            q_start.append(row); seq_lens.append(0); state_slots.append(-1)
+        q_start_v[:] = q_start
+        seq_lens_v[:] = seq_lens
+        state_v[:] = state_slots
+        if "extra" in offs:
+            ex = view("extra")
+            ex[:len(extra)] = extra
+            ex[len(extra):] = 0
+        meta.update(q_start=q_start, seq_lens=seq_lens, state_slots=state_slots)
+
+
 class StepRunner:
     def __init__(self, model: CausalLM, cache: DeviceCache, use_graphs: bool = False, max_graph_batch: int = 256):
         self.model = model
         self.cache = cache
         self.device = model.device
         self.arena = Arena(self.device)
+        self.packer = StepPacker(cache.manager, len(cache.groups), cache.page_size)
+        self._layout, self._fill = self.packer.layout, self.packer.fill
         self._staging: Optional[torch.Tensor] = None     # pinned host buffer for the step's integers
         self._staging_dev: Optional[torch.Tensor] = None
         self._copied = None
@@ -160,111 +276,6 @@ class StepRunner:
             for e in entries:
                 mgr.commit(e.rid)
         return logits, ctx
-
-    # ---- packing the step's integers -----------------------------------------------------------
-    def _layout(self, entries, order, pad_to, max_blocks, extra):
-        """Where each array of the step lies in its one buffer of integers: tokens, where a token
-        comes from, positions, sequence ids, row starts, lengths, state slots, wanted rows, then
-        per cache group the cache row of every token and the block tables, then ``extra``.  With
-        ``pad_to`` the step is filled up with empty one-token sequences (length 0, no cache row),
-        so that its shape is fixed."""
-        mgr = self.cache.manager
-        S_real = len(entries)
-        n_pad = 0 if pad_to is None else pad_to - S_real
-        N = sum(len(e.tokens) for e in entries) + n_pad
-        S = S_real + n_pad
-        R = sum(len(e.want) for e in entries) + n_pad
-        G = len(self.cache.groups)
-        if max_blocks is None:
-            max_blocks = max(1, max(len(mgr.table(e.rid, g)) for e in entries for g in range(G))) if G else 1
-        n_extra = 0 if not extra else len(extra) + RECORD_WORDS * n_pad
-        offs = {}
-        o = 0
-        for name, n in (("tokens", N), ("token_src", N), ("positions", N), ("seq_of", N), ("q_start", S + 1),
-                        ("seq_lens", S), ("state_slots", S), ("want", R)):
-            offs[name] = (o, n)
-            o += n
-        for g in range(G):
-            offs[f"slot_map{g}"] = (o, N)
-            offs[f"block_table{g}"] = (o + N, S * max_blocks)
-            o += N + S * max_blocks
-        if n_extra:
-            offs["extra"] = (o, n_extra)
-            o += n_extra
-        meta = dict(N=N, S=S, R=R, G=G, max_blocks=max_blocks, n_pad=n_pad,
-                    n_decode=sum(1 for e in entries if len(e.tokens) == 1) + n_pad)
-        return offs, meta, o
-
-    def _fill(self, buf, offs, meta, entries, order, starts, extra):
-        """Write the step's integers into ``buf`` (a numpy view of pinned memory).  Long portions
-        are written as arrays, single tokens as scalars."""
-        mgr = self.cache.manager
-        ps = self.cache.page_size
-
-        def view(name):
-            a, n = offs[name]
-            return buf[a:a + n]
-        tok, src, pos, seq = view("tokens"), view("token_src"), view("positions"), view("seq_of")
-        q_start_v, seq_lens_v, state_v, want_v = view("q_start"), view("seq_lens"), view("state_slots"), view("want")
-        G, mb, n_pad = meta["G"], meta["max_blocks"], meta["n_pad"]
-        sms = [view(f"slot_map{g}") for g in range(G)]
-        bts = [view(f"block_table{g}") for g in range(G)]
-        for bt in bts:
-            bt[:] = -1
-        q_start, seq_lens, state_slots = [0], [], []
-        row0 = {}
-        row = 0
-        for s, i in enumerate(order):
-            e = entries[i]
-            n = len(e.tokens)
-            st = starts[e.rid]
-            row0[i] = row
-            if n == 1:
-                tok[row] = e.tokens[0]
-                src[row] = -1 if e.from_sampled is None else e.from_sampled
-                pos[row] = st
-                seq[row] = s
-            else:
-                tok[row:row + n] = e.tokens
-                src[row:row + n] = -1
-                pos[row:row + n] = np.arange(st, st + n, dtype=np.int32)
-                seq[row:row + n] = s
-            for g in range(G):
-                t = mgr.table(e.rid, g)
-                if n == 1:
-                    page = t[st // ps]
-                    if page < 0:
-                        raise StepError(f"position {st} of {e.rid!r} lies in a page that was given back")
-                    sms[g][row] = page * ps + st % ps
-                else:
-                    sms[g][row:row + n] = mgr.slots_for(e.rid, g, st, n)
-                bts[g][s * mb:s * mb + len(t)] = t
-            row += n
-            q_start.append(row)
-            seq_lens.append(st + n)
-            state_slots.append(mgr.state_slot(e.rid))
-        S_real = len(entries)
-        r = 0
-        for i, e in enumerate(entries):
-            for w in e.want:
-                want_v[r] = row0[i] + int(w)
-                r += 1
-        for k in range(n_pad):          # empty one-token sequences
-            tok[row] = 0; src[row] = -1; pos[row] = 0; seq[row] = S_real + k
-            for g in range(G):
-                sms[g][row] = -1
-            want_v[r] = row
-            r += 1
-            row += 1
-            q_start.append(row); seq_lens.append(0); state_slots.append(-1)
-        q_start_v[:] = q_start
-        seq_lens_v[:] = seq_lens
-        state_v[:] = state_slots
-        if "extra" in offs:
-            ex = view("extra")
-            ex[:len(extra)] = extra
-            ex[len(extra):] = 0
-        meta.update(q_start=q_start, seq_lens=seq_lens, state_slots=state_slots)
 
     def _context(self, dev, offs, meta, arena) -> StepContext:
         def view(name):
