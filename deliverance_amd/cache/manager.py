@@ -19,7 +19,7 @@ between requests.  Here a pool of fixed size serves all requests:
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -111,6 +111,8 @@ class CacheManager:
         self._free_slots: List[int] = list(range(n_state_slots - 1, -1, -1))
         self._slot_owner: List[Optional[Hashable]] = [None] * n_state_slots
         self._reqs: Dict[Hashable, _Request] = {}
+        # called with (group, pages) whenever pages go back to a pool (a debug run poisons them)
+        self.on_release: Optional[Callable[[int, Sequence[int]], None]] = None
 
     # ---- requests ----------------------------------------------------------------
     def __contains__(self, rid) -> bool:
@@ -190,6 +192,11 @@ class CacheManager:
         r.pending += n_new
         return start
 
+    def _give(self, group: int, pages: Sequence[int], rid) -> None:
+        self.pools[group].give(pages, rid)
+        if pages and self.on_release is not None:
+            self.on_release(group, pages)
+
     def commit(self, rid, n: Optional[int] = None) -> List[Tuple[int, int]]:
         """The reserved positions (the first ``n`` of them, when given: a later step may have
         reserved more already) now belong to the request.  Pages that every later query
@@ -206,7 +213,7 @@ class CacheManager:
             t = r.tables[g]
             for j in range(min(first, len(t))):
                 if t[j] >= 0:
-                    pool.give([t[j]], rid)
+                    self._give(g, [t[j]], rid)
                     released.append((g, t[j]))
                     t[j] = -1
         return released
@@ -218,15 +225,15 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             t = r.tables[g]
             extra = [p for p in t[keep:] if p >= 0]
-            pool.give(extra, rid)
+            self._give(g, extra, rid)
             del t[keep:]
         r.pending = 0
 
     def close(self, rid) -> None:
         """End of a request: every page and the state slot go back."""
         r = self._req(rid)
-        for g, pool in enumerate(self.pools):
-            pool.give([p for p in r.tables[g] if p >= 0], rid)
+        for g in range(len(self.pools)):
+            self._give(g, [p for p in r.tables[g] if p >= 0], rid)
         if r.state_slot >= 0:
             if self._slot_owner[r.state_slot] != rid:
                 raise CacheError(f"state slot {r.state_slot} is not held by {rid!r}")

@@ -20,7 +20,7 @@ from ..parts.base import KVNeed, StateNeed
 
 class DeviceCache:
     def __init__(self, needs: Dict[int, object], dtype: torch.dtype, device, page_size: int,
-                 max_cached_tokens: int, n_state_slots: int):
+                 max_cached_tokens: int, n_state_slots: int, poison_freed: bool = False):
         self.dtype = dtype
         self.device = torch.device(device)
         self.page_size = page_size
@@ -55,6 +55,14 @@ class DeviceCache:
             self.state[s.slot] = torch.zeros((n_slots, s.elems), dtype=torch.float32, device=self.device)
         self.manager = CacheManager(self.groups, page_size, [self.n_pages] * len(self.groups),
                                     state_specs, n_slots)
+        if poison_freed:
+            # debug runs: a page that goes back is filled with NaN again (after the steps that were
+            # launched before, in stream order), so that a row read before its new owner wrote it shows
+            self.manager.on_release = self._poison
+
+    def _poison(self, group: int, pages) -> None:
+        idx = torch.tensor(list(pages), dtype=torch.long, device=self.device)
+        self._group_tensors[group].index_fill_(1, idx, float("nan"))
 
     def reset_state(self, state_slot: int) -> None:
         """A request that starts gets a zeroed state row in every state tensor."""

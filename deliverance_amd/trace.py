@@ -24,7 +24,8 @@ import sys
 class TraceSession:
     """The engine's model, cache and step function, driven one trace step at a time."""
 
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0"):
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
+                 poison_freed: bool = False):
         import torch
         from . import models  # noqa: F401  (registers the architectures)
         from .engine.device_cache import DeviceCache
@@ -37,7 +38,7 @@ class TraceSession:
         # A request's count is rounded up to a multiple of 64, so max_tokens / page_size pages
         # hold every live request whatever its length.
         self.cache = DeviceCache(self.model.cache_needs(), tdtype, device, page_size, max(max_tokens, 64),
-                                 n_state_slots=8)
+                                 n_state_slots=8, poison_freed=poison_freed)
         self.runner = StepRunner(self.model, self.cache)
 
     def run_step(self, rec: dict):

@@ -142,3 +142,27 @@ def test_random_orders_keep_every_invariant(seed):
         m.close(rid)
     m.check()
     assert [p.n_free for p in m.pools] == [n_pages, n_pages]
+
+
+def test_release_hook_sees_every_page_that_goes_back():
+    """close, rollback and the window's release all report the pages they give back (a debug run
+    fills them with NaN on the device)."""
+    mgr = CacheManager([KVGroupSpec((0,), 1, 16, None), KVGroupSpec((1,), 1, 16, 20)], 16, [8, 8])
+    seen = []
+    mgr.on_release = lambda g, pages: seen.append((g, list(pages)))
+    mgr.open("a")
+    mgr.extend("a", 40)
+    released = mgr.commit("a")                       # the window of 20 has passed page 0 of group 1
+    assert seen == [(g, [p]) for g, p in released] and [g for g, _ in seen] == [1]
+    seen.clear()
+    mgr.extend("a", 30)
+    before = {g: list(mgr.table("a", g)) for g in (0, 1)}
+    mgr.rollback("a")
+    after = {g: list(mgr.table("a", g)) for g in (0, 1)}
+    assert sorted(p for g, ps in seen for p in ps if g == 0) == sorted(set(before[0]) - set(after[0]))
+    seen.clear()
+    held = {g: [p for p in mgr.table("a", g) if p >= 0] for g in (0, 1)}
+    mgr.close("a")
+    assert {g: ps for g, ps in seen} == held
+    mgr.check()
+    assert all(pool.n_free == 8 for pool in mgr.pools)

@@ -19,7 +19,7 @@ LENGTHS = {"A": (5, 17, 40, 56), "B": (1, 9, 33, 64, 88)}
 
 def session_for(model, dtype, max_tokens, page_size=16):
     from deliverance_amd.trace import TraceSession
-    return TraceSession(model.folder, dtype, max_tokens, page_size)
+    return TraceSession(model.folder, dtype, max_tokens, page_size, poison_freed=True)   # pages that go back are NaN again
 
 
 def requests_of(model, name):

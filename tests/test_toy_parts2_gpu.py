@@ -204,7 +204,7 @@ def test_window_groups_rotation_and_routing_through_the_engine(toy_folder, dtype
     from deliverance_amd.parts import KVNeed
     from deliverance_amd.trace import TraceSession
     _, W = P.read_model_folder(toy_folder)
-    s = TraceSession(toy_folder, dtype, 512)
+    s = TraceSession(toy_folder, dtype, 512, poison_freed=True)     # pages that the window has passed are NaN again
     needs = s.model.cache_needs()
     assert needs[0] == KVNeed(HKV0, D0, WINDOW) and needs[1] == KVNeed(HKV1, D1, None)
     assert len(s.cache.groups) == 2                         # pages of their own for the two layers

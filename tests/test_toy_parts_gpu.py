@@ -155,7 +155,7 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_folder, dtype):
     from deliverance_amd.parts import KVNeed, StateNeed
     from deliverance_amd.trace import TraceSession
     _, W = P.read_model_folder(toy_folder)
-    s = TraceSession(toy_folder, dtype, 256)
+    s = TraceSession(toy_folder, dtype, 256, poison_freed=True)
     needs = s.model.cache_needs()
     assert isinstance(needs[0], KVNeed) and isinstance(needs[1], StateNeed) and isinstance(needs[2], KVNeed)
     assert needs[1].elems == E + 1 and set(s.cache.state) == {1}
