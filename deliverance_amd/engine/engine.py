@@ -74,7 +74,8 @@ class CausalLanguageModel:
             tokens = min(tokens, engine_config.max_num_seqs * model.config.max_positions)
             tokens = max(tokens, engine_config.page_size)
         n_slots = engine_config.state_slots if engine_config.state_slots is not None else engine_config.max_num_seqs
-        self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots)
+        self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots,
+                                 poison_freed=engine_config.poison_freed_pages)
         self.runner = StepRunner(model, self.cache, use_graphs=engine_config.use_graphs,
                                  max_graph_batch=max(engine_config.max_num_seqs, 1))
         self.scheduler = Scheduler(self.cache.manager, model.config.max_positions, model.config.eos_token_ids,

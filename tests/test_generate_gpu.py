@@ -162,7 +162,8 @@ def test_when_pages_run_out_requests_are_computed_again_with_the_same_result(mod
     params = GeneratorParameters(max_tokens=40, ignore_eos=True)
     roomy = load(m, dtype, max_cached_tokens=1024)
     want = [o.generated_tokens for o in roomy.generate(prompts, params)]
-    tight = load(m, dtype, max_cached_tokens=192, max_batch_tokens=48, max_chunk=16)    # 12 pages for ~270 tokens
+    tight = load(m, dtype, max_cached_tokens=192, max_batch_tokens=48, max_chunk=16,     # 12 pages for ~270 tokens
+                 poison_freed_pages=True)      # and what a request that is set back gives up is NaN again
     outs = tight.generate(prompts, params)
     assert sum(o.preemptions for o in outs) >= 1 and tight.stats()["preemptions"] >= 1
     if dtype == "float32":
