@@ -9,6 +9,7 @@ library and without ``hipcc`` the engine refuses to run.
 from __future__ import annotations
 
 import ctypes
+import fcntl
 import glob
 import hashlib
 import os
@@ -106,6 +107,18 @@ def build(force: bool = False, verbose: bool = True) -> str:
     srcs = _sources()
     if not srcs:
         raise KernelLibraryError(f"no HIP sources under {CSRC}")
+    # one build at a time per folder: processes that start together in a fresh checkout would
+    # otherwise write the same object files; whoever waited finds the library built
+    with open(os.path.join(out_dir, ".build.lock"), "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        if not force:
+            p = library_path()
+            if p:
+                return p
+        return _build_locked(hipcc, out_dir, srcs, verbose)
+
+
+def _build_locked(hipcc: str, out_dir: str, srcs, verbose: bool) -> str:
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)       # hipcc wants somewhere to keep its temporary files
     env.setdefault("TMPDIR", tempfile.gettempdir())
