@@ -71,9 +71,10 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
 
   // Loads are never conditional (a conditional load becomes a branch that serialises the slab's
   // loads).  Rows past the edge of a or w read the last row instead: what they produce is never
-  // stored.  Chunks past K (KTAIL: K is no multiple of the slab) read chunk 0 and are replaced by
-  // zero afterwards; that replacement makes the compiler wait for loads early, so it is compiled
-  // only where it is needed.  PF_SLABS slabs are in flight in registers at any time: one slab's
+  // stored.  Chunks past K (KTAIL: K is no multiple of the slab) read the row's first chunk and are
+  // replaced by zero afterwards; that replacement makes the compiler wait for loads early, so it is
+  // compiled only where it is needed.  (The row's first chunk, not this thread's chunk of slab 0:
+  // with K < 64 that one lies past K too, in the next row or, for the last row, past the tensor.)  PF_SLABS slabs are in flight in registers at any time: one slab's
   // products take far less time than a load, so the distance between asking and needing is what
   // keeps the matrix cores fed.
   uint4 ra[PF_SLABS][CA], rw[PF_SLABS][CW];
@@ -94,7 +95,7 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
 #define TILE_FETCH(stage, k0)                                   \
   {                                                             \
     const bool kin = !KTAIL || (k0) + kc_t < K;                 \
-    const int ks = kin ? (k0) : 0;                              \
+    const int ks = kin ? (k0) : -kc_t;                          \
     _Pragma("unroll") for (int i = 0; i < CA; ++i) {            \
       ra[stage][i] = load16(pa[i] + ks);                        \
       if (KTAIL && !kin) ra[stage][i] = zero;                   \

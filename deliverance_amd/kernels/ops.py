@@ -276,7 +276,7 @@ def _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, name):
     _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
           f"{name}: slot_map must be int32 [rows]")
     _need(q_cols + 2 * Hkv * D == N, f"{name}: q|k|v columns do not add up to N")
-    return kv_cache.data_ptr(), slot_map.data_ptr(), q_cols, Hkv * D, Hkv, D, page
+    return _ptr(kv_cache), _ptr(slot_map), q_cols, Hkv * D, Hkv, D, page
 
 
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,

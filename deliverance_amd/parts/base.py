@@ -163,9 +163,16 @@ build_feed_forward = _build(_FEED_FORWARDS, "feed-forward")
 build_position = _build(_POSITIONS, "position encoding")
 
 
+def _owned(out: torch.Tensor, src: torch.Tensor) -> torch.Tensor:
+    """A part owns its parameters: when the conversion was a no-op, ``out`` still is the caller's
+    memory (a mapped checkpoint file, read-only and at any alignment, or a tensor the caller may
+    change), so it is copied."""
+    return out.clone() if out.data_ptr() == src.data_ptr() else out
+
+
 def to_matrix(t: torch.Tensor, dtype: torch.dtype, device) -> torch.Tensor:
     """A matrix operand of the compute dtype on the device ([out, in], contiguous)."""
-    return t.to(device=device, dtype=dtype).contiguous()
+    return _owned(t.to(device=device, dtype=dtype).contiguous(), t)
 
 
 def to_vector(t: Optional[torch.Tensor], dtype: torch.dtype, device) -> Optional[torch.Tensor]:
@@ -173,7 +180,8 @@ def to_vector(t: Optional[torch.Tensor], dtype: torch.dtype, device) -> Optional
     if t is None:
         return None
     if dtype == torch.float32:
-        return t.to(device=device, dtype=torch.float32).contiguous()
+        return _owned(t.to(device=device, dtype=torch.float32).contiguous(), t)
+    src = t
     if t.dtype not in (torch.bfloat16, torch.float32):
         t = t.to(torch.float32)
-    return t.to(device=device).contiguous()
+    return _owned(t.to(device=device).contiguous(), src)

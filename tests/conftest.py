@@ -9,12 +9,25 @@ for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
         sys.path.insert(0, p)
 
 
+# With DELIVERANCE_SIMT=1 the GPU tests that drive kernels, parts and trace sessions run on the CPU
+# instead: the kernels compiled for the host, every operand of every kernel call between protected
+# pages (tests/simt).  tests/test_simt.py starts such runs as child processes.
+SIMT = os.environ.get("DELIVERANCE_SIMT") == "1"
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "needs_device: a GPU test that cannot run on the simulated kernels")
 
 
 def pytest_collection_modifyitems(config, items):
     """GPU tests are skipped where no GPU is visible, so a plain `pytest tests` passes on a CPU box."""
+    if SIMT:
+        skip = pytest.mark.skip(reason="needs the device itself (streams, graphs, pinned memory)")
+        for item in items:
+            if "needs_device" in item.keywords:
+                item.add_marker(skip)
+        return
     try:
         import torch
         have = torch.cuda.is_available()
@@ -26,6 +39,16 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _simulated_kernels():
+    if not SIMT:
+        yield
+        return
+    from simt import harness
+    with harness.Sim().patched(auto_guard=True):
+        yield
 
 
 @pytest.fixture(scope="session")

@@ -18,6 +18,27 @@ CONFIG_B = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=3,
                 activation_function="gelu", scale_attn_by_inverse_layer_idx=True, bos_token_id=0,
                 eos_token_id=999)
 
+# Where the GPU tests put their tensors: the GPU, or (DELIVERANCE_SIMT=1) the CPU, where the kernels
+# run simulated under guard pages (tests/simt).
+SIMT = os.environ.get("DELIVERANCE_SIMT") == "1"
+DEVICE = "cpu" if SIMT else "cuda:0"
+
+
+def trace_session(folder, dtype, max_tokens, page_size=16, poison_freed=False):
+    """The engine's trace session on the GPU, or its stand-in on the simulated kernels."""
+    if SIMT:
+        from simt import harness
+        return harness.SimTraceSession(None, str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed)
+    from deliverance_amd.trace import TraceSession
+    return TraceSession(str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed)
+
+
+def skip_in_simulation_if(cond, why="too much arithmetic for the simulated kernels"):
+    if SIMT and cond:
+        import pytest
+        pytest.skip(why)
+
+
 # Absolute tolerances on logits (their magnitude is about 1 on these models).
 ATOL = {"float32": 5e-6, "bfloat16": 1.5e-2}
 

@@ -8,10 +8,11 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+import helpers
 import plain_gpt2 as P
 
 pytestmark = pytest.mark.gpu
-DEV = "cuda:0"
+DEV = helpers.DEVICE
 
 
 @pytest.fixture(scope="module")
@@ -106,6 +107,7 @@ def test_gemm_matrix_cores(ops, M, N, K):
     wavefronts; up to 64 rows: 16x16x32 products fed through LDS, 1 to 4 row tiles, 8 or 12 wavefronts;
     else block tiles of 64x64, 128x64 and 128x128, chosen by the number of tiles: 1,100 and 2,048 rows
     reach the larger ones), each with a last step that K cuts."""
+    helpers.skip_in_simulation_if(M * N * K > 1.2e8)
     g = torch.Generator().manual_seed(M * 7 + N)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
                                (None, True, True, torch.float32), (None, False, False, torch.float32),
@@ -425,6 +427,7 @@ def test_xtc_and_logprobs(ops):
                                    (5, 64, 1304), (2, 48, 8), (11, 200, 1992)])
 @pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_product(ops, M, N, K, pdtype):
+    helpers.skip_in_simulation_if(M * N * K > 1.2e8)
     g = torch.Generator().manual_seed(M + N)
     x = (torch.randn(M + 3, K, generator=g) * 2 + 1).to(DEV)
     gw, gb = torch.randn(K, generator=g).to(pdtype).to(DEV), torch.randn(K, generator=g).to(pdtype).to(DEV)

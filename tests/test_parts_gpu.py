@@ -7,10 +7,11 @@ import numpy as np
 import pytest
 import torch
 
+import helpers
 import plain_gpt2 as P
 
 pytestmark = pytest.mark.gpu
-DEV = "cuda:0"
+DEV = helpers.DEVICE
 TOL = {torch.float32: 3e-5, torch.bfloat16: 4e-2}
 
 

@@ -2,17 +2,19 @@
 widths that are no multiple of 8, odd vocabularies, every page size, every activation) replayed
 mixed, with pages used again, and whole, against the plain implementation, in 32-bit and in
 bfloat16: a size that a kernel does not take must be refused or served by another kernel, never
-answered wrongly."""
+answered wrongly.
+
+Seeds 5 and 11 hold products whose inner size is 32, below one 64-wide slab of the block-tile
+kernel: its loads past K once fell back to an address that was itself past K (the thread's own
+chunk of the first slab, not the row's first chunk) and read up to 64 bytes behind the last row of
+an operand, which faults only when the operand ends where mapped memory ends.  tests/test_simt.py
+runs these two seeds on the CPU with every operand between protected pages."""
 import numpy as np
 import pytest
 
 import helpers
 
-pytestmark = [pytest.mark.gpu,
-              pytest.mark.skip(reason="the one run of the whole suite that held this file (together with a variant of the "
-                                      "fused norm + product kernel that has been taken out again) ended in a GPU memory "
-                                      "fault whose cause was not found; the same traces had passed in a process of their "
-                                      "own; it stays off the GPU until the cause is known")]
+pytestmark = pytest.mark.gpu
 
 
 def draw_config(seed):
@@ -33,7 +35,6 @@ def draw_config(seed):
 # seeds chosen so that the head sizes 16, 32, 80, 96, 112, 128, 160 and 256 all occur
 @pytest.mark.parametrize("seed", [1, 4, 5, 7, 11, 13, 212, 218])
 def test_random_configuration_mixed_and_whole(tmp_path, seed):
-    from deliverance_amd.trace import TraceSession
     cfg, page, rng = draw_config(seed)
     m = helpers.make_model(tmp_path, cfg, seed)
     P = cfg["n_positions"]
@@ -42,11 +43,11 @@ def test_random_configuration_mixed_and_whole(tmp_path, seed):
     steps = helpers.trace_mixed(reqs, seed=seed, prefill_sizes=(9, 2, 67, 4, 130, 33), decode_tail=int(rng.integers(1, 20)))
     unit = max(64, page)
     for dtype in ("float32", "bfloat16"):
-        s = TraceSession(m.folder, dtype, helpers.max_live_tokens(steps, round_to=unit), page)
+        s = helpers.trace_session(m.folder, dtype, helpers.max_live_tokens(steps, round_to=unit), page)
         got = helpers.replay(s, steps)
         helpers.check_against_plain(m, got, reqs, dtype, f"mixed {cfg} page {page}")
         s.cache.manager.check()
         assert s.cache.manager.pools[0].n_free == s.cache.n_pages
-        s = TraceSession(m.folder, dtype, -(-P // unit) * unit, page)
+        s = helpers.trace_session(m.folder, dtype, -(-P // unit) * unit, page)
         got = helpers.replay(s, helpers.trace_whole(*reqs[-1]))
         helpers.check_against_plain(m, got, reqs[-1:], dtype, f"whole {cfg} page {page}")

@@ -18,8 +18,7 @@ LENGTHS = {"A": (5, 17, 40, 56), "B": (1, 9, 33, 64, 88)}
 
 
 def session_for(model, dtype, max_tokens, page_size=16):
-    from deliverance_amd.trace import TraceSession
-    return TraceSession(model.folder, dtype, max_tokens, page_size, poison_freed=True)   # pages that go back are NaN again
+    return helpers.trace_session(model.folder, dtype, max_tokens, page_size, poison_freed=True)   # pages that go back are NaN again
 
 
 def requests_of(model, name):
@@ -188,6 +187,7 @@ def test_errors_leave_the_cache_as_it_was(model_a):
     assert s.cache.manager.live() == [] and s.cache.manager.pools[0].n_free == 4
 
 
+@pytest.mark.needs_device
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_bin_trace_run(model_b, dtype, tmp_path):
     """The program itself: steps on stdin, `done <step>` lines, <step>.f32 files."""

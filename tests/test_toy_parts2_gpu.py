@@ -202,9 +202,8 @@ def toy_folder(tmp_path_factory):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_window_groups_rotation_and_routing_through_the_engine(toy_folder, dtype):
     from deliverance_amd.parts import KVNeed
-    from deliverance_amd.trace import TraceSession
     _, W = P.read_model_folder(toy_folder)
-    s = TraceSession(toy_folder, dtype, 512, poison_freed=True)     # pages that the window has passed are NaN again
+    s = helpers.trace_session(toy_folder, dtype, 512, poison_freed=True)     # pages that the window has passed are NaN again
     needs = s.model.cache_needs()
     assert needs[0] == KVNeed(HKV0, D0, WINDOW) and needs[1] == KVNeed(HKV1, D1, None)
     assert len(s.cache.groups) == 2                         # pages of their own for the two layers
@@ -241,6 +240,7 @@ def test_window_groups_rotation_and_routing_through_the_engine(toy_folder, dtype
     assert s.cache.manager.live() == []
 
 
+@pytest.mark.needs_device
 def test_generation_with_the_toy_parts(toy_folder):
     from deliverance_amd import AutoModelForCausalLM, GeneratorParameters
     _, W = P.read_model_folder(toy_folder)

@@ -153,9 +153,8 @@ def toy_folder(tmp_path_factory):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_architecture_is_registered_built_and_stepped(toy_folder, dtype):
     from deliverance_amd.parts import KVNeed, StateNeed
-    from deliverance_amd.trace import TraceSession
     _, W = P.read_model_folder(toy_folder)
-    s = TraceSession(toy_folder, dtype, 256, poison_freed=True)
+    s = helpers.trace_session(toy_folder, dtype, 256, poison_freed=True)
     needs = s.model.cache_needs()
     assert isinstance(needs[0], KVNeed) and isinstance(needs[1], StateNeed) and isinstance(needs[2], KVNeed)
     assert needs[1].elems == E + 1 and set(s.cache.state) == {1}
@@ -181,6 +180,7 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_folder, dtype):
     assert np.array_equal(a, b)
 
 
+@pytest.mark.needs_device
 def test_toy_architecture_generates_through_the_entry_point(toy_folder):
     from deliverance_amd import AutoModelForCausalLM, GeneratorParameters
     _, W = P.read_model_folder(toy_folder)
@@ -206,10 +206,10 @@ def test_run_order_mistakes_are_refused(toy_folder):
     t = load_declared(toy_folder, arch.declare_tensors(mc))
     bad = dataclasses.replace(mc, schedule=(LayerCall(0, 0, True), LayerCall(2, 0, True)))
     with pytest.raises(ValueError, match="written by two"):
-        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, "cuda:0").cache_needs()
+        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, helpers.DEVICE).cache_needs()
     bad = dataclasses.replace(mc, schedule=(LayerCall(0, 0, True), LayerCall(2, 5, False)))
     with pytest.raises(ValueError, match="nothing writes"):
-        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, "cuda:0").cache_needs()
+        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, helpers.DEVICE).cache_needs()
     bad = dataclasses.replace(mc, schedule=(LayerCall(0, 0, True), LayerCall(7, 1, True)))
     with pytest.raises(ValueError, match="run order names layer 7"):
-        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, "cuda:0")
+        CausalLM(bad, arch.bind_tensors(bad, t), torch.float32, helpers.DEVICE)
