@@ -1,6 +1,6 @@
 """Command line.  Option names and meanings follow the reference's benchmark main where it has
 them (core/src/main/java/io/teknek/deliverance/benchmark/InferenceBenchmark.java:1036-1141):
-``--model``, ``--working-dtype``, ``--max-tokens`` (256), ``--temperature`` (0.0), ``--seed N|none``
+``--model``, ``--working-dtype``, ``--kernels`` (the reference's ``--tensor-provider``), ``--max-tokens`` (256), ``--temperature`` (0.0), ``--seed N|none``
 (42), ``--warmup-cases`` (1), ``--max-cases``, ``--kv-context-rows-per-page``, ``--model-config``,
 ``--profile-stages``, ``--suite-file``, ``--output`` (CSV), ``--jsonl-output``.  The engine works
 on token ids, so prompts are lists of ids (``--prompt-ids 5,17,3`` or a JSONL suite file with a
@@ -53,7 +53,7 @@ def cmd_generate(a) -> int:
     if a.model_config:
         with open(a.model_config) as f:
             cfg = json.load(f)
-    cfg.update({k: v for k, v in dict(dtype=a.working_dtype, page_size=a.kv_context_rows_per_page,
+    cfg.update({k: v for k, v in dict(dtype=a.working_dtype, kernels=a.kernels, page_size=a.kv_context_rows_per_page,
                                       max_batch_tokens=a.max_batch_tokens, max_num_seqs=a.max_num_seqs,
                                       max_cached_tokens=a.max_cached_tokens).items() if v is not None})
     if a.profile_stages:
@@ -139,6 +139,9 @@ def main(argv=None) -> int:
     g = sub.add_parser("generate", help="generate tokens for prompts of token ids")
     g.add_argument("--model", required=True, help="model folder (config.json + safetensors)")
     g.add_argument("--working-dtype", type=_dtype_name, default=None, help="BF16 (default) or F32")
+    g.add_argument("--kernels", choices=["tuned", "reference"], default=None,
+                   help="bfloat16: the serving kernels (default) or the plain kernels, as the reference's "
+                        "--tensor-provider picks its math")
     g.add_argument("--prompt-ids", action="append", help="comma-separated token ids; may be given several times")
     g.add_argument("--suite-file", help="JSONL, one object with a prompt_ids list per line")
     g.add_argument("--max-tokens", type=int, default=256, help="max generated tokens per prompt, default 256")

@@ -13,10 +13,28 @@ DTYPE_NAMES = {"bfloat16": "bfloat16", "bf16": "bfloat16", "BF16": "bfloat16",
                "float32": "float32", "fp32": "float32", "f32": "float32", "F32": "float32"}
 
 
+KERNEL_MODES = ("tuned", "reference")
+PAGE_SIZES = (16, 32, 64)
+
+
+def check_page_size(page_size: int) -> int:
+    """The page sizes every attention kernel takes (the bfloat16 kernels walk keys in aligned runs of
+    64); refused here, before anything is reserved, rather than at the first launch."""
+    if page_size not in PAGE_SIZES:
+        raise ValueError(f"page_size must be one of {PAGE_SIZES}, found {page_size}")
+    return page_size
+
+
 @dataclass
 class EngineConfig:
     dtype: str = "bfloat16"            # "bfloat16" (serving kernels) or "float32" (true 32-bit)
-    page_size: int = 16                # tokens per KV page; a multiple of 16
+    # "tuned": matrix-core products and the prefill/decode attention kernels in bfloat16; "reference":
+    # the plain kernels in bfloat16 too, which splits a mismatch into "tuned kernel" or "bfloat16
+    # rounding" (the reference picks its math provider in the same place:
+    # core/src/main/java/io/teknek/deliverance/benchmark/InferenceBenchmark.java:1067,1139).
+    # 32-bit always runs the plain kernels.
+    kernels: str = "tuned"
+    page_size: int = 16                # tokens per KV page: 16, 32 or 64 (what every attention kernel takes)
     max_cached_tokens: Optional[int] = None   # pool size in tokens; None: sized from free memory
     max_num_seqs: int = 64             # live requests at a time
     max_batch_tokens: int = 2048       # token budget of one step
@@ -31,7 +49,8 @@ class EngineConfig:
         if self.dtype not in DTYPE_NAMES:
             raise ValueError(f"dtype must be bfloat16 or float32, found {self.dtype!r}")
         self.dtype = DTYPE_NAMES[self.dtype]
-        if self.page_size <= 0 or self.page_size % 16 != 0:
-            raise ValueError(f"page_size must be a positive multiple of 16, found {self.page_size}")
+        if self.kernels not in KERNEL_MODES:
+            raise ValueError(f"kernels must be one of {KERNEL_MODES}, found {self.kernels!r}")
+        check_page_size(self.page_size)
         if self.max_num_seqs <= 0 or self.max_batch_tokens <= 0 or self.max_chunk <= 0:
             raise ValueError("max_num_seqs, max_batch_tokens and max_chunk must be positive")

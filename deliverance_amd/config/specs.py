@@ -110,6 +110,7 @@ class ModelConfig:
     bos_token_id: Optional[int]
     eos_token_ids: Tuple[int, ...]
     raw: dict = field(default_factory=dict, compare=False, hash=False)
+    embed_scale: float = 1.0        # multiplies the token embedding before positions are added
 
     @property
     def n_cache_slots(self) -> int:

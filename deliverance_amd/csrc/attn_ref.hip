@@ -57,7 +57,9 @@ attn_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache,
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float e = valid ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);      // 0 on the first chunk (m = -inf)
+    // 0 on the first chunk that shows a key (m = -inf); 1 while no key has been seen at all (a
+    // padding row of a fixed-shape step: -inf - -inf would be NaN, and NaN * 0 stays NaN)
+    const float alpha = m_new == -INFINITY ? 1.f : expf(m - m_new);
     l = l * alpha + wave_sum(e);
     m = m_new;
     ps[lane] = e;

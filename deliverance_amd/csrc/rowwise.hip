@@ -15,31 +15,61 @@ void da_set_error(const char* fmt, ...) {
 }
 
 // ------------------------------------------------------------------------------------------
-// x[n, :] = wte[token[n], :] + wpe[pos[n], :]      (32-bit sum, 32-bit result)
+// x[n, :] = wte[token[n], :] * scale + wpe[pos[n], :]      (32-bit sum, 32-bit result)
 // Reference: core/src/main/java/io/teknek/deliverance/model/gpt2/Gpt2Model.java:42-48
+// (GPT-2: scale 1; the factor is there for architectures that multiply their embeddings).
 // ------------------------------------------------------------------------------------------
 __global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
                              const void* __restrict__ wte, int wte_dtype,
                              const void* __restrict__ wpe, int wpe_dtype,
-                             float* __restrict__ x, int E) {
+                             float* __restrict__ x, int E, float scale) {
   const int n = blockIdx.x;
   const size_t trow = (size_t)tokens[n] * E;
   const size_t prow = wpe ? (size_t)positions[n] * E : 0;
   for (int i = threadIdx.x; i < E; i += blockDim.x) {
     float v = load_param(wte, wte_dtype, trow + i);
+    if (scale != 1.0f) v *= scale;
     if (wpe) v += load_param(wpe, wpe_dtype, prow + i);
     x[(size_t)n * E + i] = v;
   }
 }
 
 extern "C" int da_embed(const int* tokens, const int* positions, const void* wte, int wte_dtype,
-                        const void* wpe, int wpe_dtype, float* x, int N, int E, void* stream) {
+                        const void* wpe, int wpe_dtype, float* x, int N, int E, float scale, void* stream) {
   DA_REQUIRE(N >= 0 && E > 0, "embed: bad sizes N=%d E=%d", N, E);
   if (N == 0) return 0;
   int threads = E >= 256 ? 256 : (E >= 128 ? 128 : 64);
   hipLaunchKernelGGL(embed_kernel, dim3(N), dim3(threads), 0, (hipStream_t)stream, tokens, positions,
-                     wte, wte_dtype, wpe, wpe_dtype, x, E);
+                     wte, wte_dtype, wpe, wpe_dtype, x, E, scale);
   DA_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// dst[r, :] (+)= src[rows ? rows[r] : r, :]: rows gathered, converted between 32-bit and
+// bfloat16, or added into the 32-bit residual stream.  For blocks without a norm in front of a
+// part, models without a final norm, and norms that follow a part.
+// ------------------------------------------------------------------------------------------
+__global__ void copy_rows_kernel(const void* __restrict__ src, int src_dtype, const int* __restrict__ rows,
+                                 void* __restrict__ dst, int dst_dtype, int E, int accumulate) {
+  const int r = blockIdx.x;
+  const size_t srow = (size_t)(rows ? rows[r] : r) * E, drow = (size_t)r * E;
+  for (int i = threadIdx.x; i < E; i += blockDim.x) {
+    const float v = load_param(src, src_dtype, srow + i);
+    if (accumulate) ((float*)dst)[drow + i] += v;
+    else store_out(dst, dst_dtype, drow + i, v);
+  }
+}
+
+extern "C" int da_copy_rows(const void* src, int src_dtype, const int* rows, void* dst, int dst_dtype, int R,
+                            int E, int accumulate, void* stream) {
+  DA_REQUIRE(R >= 0 && E > 0, "copy_rows: bad sizes R=%d E=%d", R, E);
+  DA_REQUIRE(!accumulate || dst_dtype == DA_F32, "copy_rows: accumulation needs a 32-bit destination");
+  if (R == 0) return 0;
+  const int threads = E >= 256 ? 256 : (E >= 128 ? 128 : 64);
+  hipLaunchKernelGGL(copy_rows_kernel, dim3(R), dim3(threads), 0, (hipStream_t)stream, src, src_dtype, rows, dst,
+                     dst_dtype, E, accumulate);
+  DA_CHECK_LAUNCH("copy_rows");
   return 0;
 }
 

@@ -15,6 +15,7 @@ from typing import Dict, List
 import torch
 
 from ..cache.manager import CacheManager, KVGroupSpec, StateSpec
+from ..config.engine_config import check_page_size
 from ..parts.base import KVNeed, StateNeed
 
 
@@ -23,7 +24,7 @@ class DeviceCache:
                  max_cached_tokens: int, n_state_slots: int, poison_freed: bool = False):
         self.dtype = dtype
         self.device = torch.device(device)
-        self.page_size = page_size
+        self.page_size = check_page_size(page_size)
         by_shape: Dict[tuple, List[int]] = {}
         state_specs: List[StateSpec] = []
         for slot in sorted(needs):

@@ -77,13 +77,17 @@ class CausalLanguageModel:
         self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots,
                                  poison_freed=engine_config.poison_freed_pages)
         self.runner = StepRunner(model, self.cache, use_graphs=engine_config.use_graphs,
-                                 max_graph_batch=max(engine_config.max_num_seqs, 1))
+                                 max_graph_batch=max(engine_config.max_num_seqs, 1), kernels=engine_config.kernels)
         self.scheduler = Scheduler(self.cache.manager, model.config.max_positions, model.config.eos_token_ids,
                                    engine_config.max_num_seqs, engine_config.max_batch_tokens,
                                    engine_config.max_chunk, on_open=self.cache.reset_state)
         self._next_id = 0
         self._callbacks: Dict[Hashable, Callable] = {}
         self._inflight: Optional[_InFlight] = None
+        self._ended_outside: List[Request] = []       # cancelled between steps; the next step() reports them
+        # hook(batch, logits): every launched step's scheduled portions and its logits on the device
+        # (row i: the i-th portion that samples), before anything is read back; for tests and diagnosis
+        self.logits_hook: Optional[Callable] = None
         self._n_launched = 0
         n = 2 * max(engine_config.max_num_seqs, 64)
         self._token_bufs = [torch.empty(n, dtype=torch.int32, pin_memory=True) for _ in range(3)]
@@ -103,7 +107,30 @@ class CausalLanguageModel:
         return rid
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work() or self._inflight is not None
+        return self.scheduler.has_work() or self._inflight is not None or bool(self._ended_outside)
+
+    def cancel(self, rid: Hashable) -> bool:
+        """End a request now, between two steps (also from inside an ``on_token`` callback); True when
+        it was waiting or running.  Its pages and state slot go back at once, also those that a step
+        which is still running holds for it: that step's work for the request is dropped when the
+        step is read, and whoever gets the pages next writes them after that step in stream order.
+        The request ends with ``finish_reason = "cancelled"`` and is reported by the next ``step()``.
+        The reference stops a generation between two tokens likewise
+        (core/src/main/java/io/teknek/deliverance/model/GenerationEngine.java:221-225)."""
+        before = len(self.scheduler.finished)
+        if not self.scheduler.cancel(rid):
+            return False
+        self._ended_outside += self.scheduler.finished[before:]
+        self._callbacks.pop(rid, None)
+        return True
+
+    def set_layer_debug_hook(self, hook: Optional[Callable]) -> None:
+        """``hook(layer, stage, tensor)`` receives copies of named intermediates of every step (layer -1,
+        "input": the embedding; per layer "query_projection", "key_projection", "value_projection",
+        "attention_value", "post_attention_residual", "post_ff_residual", "layer_output"), as the
+        reference's ``setLayerDebugHook`` does (core/.../model/AbstractModel.java:122-128,505-515,1100-1107).
+        While a hook is set, steps run kernel by kernel (no recorded graphs) and slowly."""
+        self.runner.debug_hook = hook
 
     def step(self) -> List[Request]:
         """One scheduler decision and one model step with its sampling.  Returns the requests
@@ -114,7 +141,8 @@ class CausalLanguageModel:
         on the device) and only then reads the older step's tokens, so the host's work for one
         step runs beside the device's work for the step before.  When the next step cannot be
         decided ahead (pages are short), the older step is read first, as without this."""
-        done: List[Request] = []
+        done: List[Request] = self._ended_outside
+        self._ended_outside = []
         if self._inflight is not None:
             ahead = self._launch_ahead(self._inflight)
             done += self._retire(self._inflight)
@@ -174,8 +202,17 @@ class CausalLanguageModel:
                 records += struct.unpack(f"<{RECORD_WORDS}i", device_record(req.params, req.rng, V))
                 samplers.append(s)
         decode_only = all(s.n == 1 for s in batch)
-        with InferenceProfiler.timer("generation.decode" if decode_only else "generation.prefill"):
-            logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
+        try:
+            with InferenceProfiler.timer("generation.decode" if decode_only else "generation.prefill"):
+                logits, ctx = self.runner.run(entries, reserved=True, sample_records=records or None)
+        except Exception as e:
+            # a step that could not be put on the device: its requests end with an error and give
+            # back what the scheduler had reserved for them
+            for s in batch:
+                self.scheduler._fail(s.request, f"the step could not be launched: {e}")
+            raise
+        if self.logits_hook is not None:
+            self.logits_hook(batch, logits)
         InferenceProfiler.counter("engine.batch_tokens", sum(s.n for s in batch))
         flight = _InFlight(batch, samplers)
         if not samplers:

@@ -122,7 +122,9 @@ class Scheduler:
         """The largest portion <= n whose pages are free right now."""
         ps = self.cache.page_size
         if opened:
-            have = len(self.cache.table(req.rid, 0)) * ps if self.cache.groups else 10 ** 9
+            # every group has a table of the same length; the smallest is what counts should they differ
+            have = min((len(self.cache.table(req.rid, g)) for g in range(len(self.cache.groups))), default=None)
+            have = 10 ** 9 if have is None else have * ps
             base = self.cache.length(req.rid) + self.cache.pending(req.rid)
         else:
             have, base = 0, 0

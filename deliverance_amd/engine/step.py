@@ -152,9 +152,14 @@ class StepPacker:
 
 
 class StepRunner:
-    def __init__(self, model: CausalLM, cache: DeviceCache, use_graphs: bool = False, max_graph_batch: int = 256):
+    def __init__(self, model: CausalLM, cache: DeviceCache, use_graphs: bool = False, max_graph_batch: int = 256,
+                 kernels: str = "tuned"):
         self.model = model
         self.cache = cache
+        self.kernels = kernels                       # "tuned" | "reference" (EngineConfig.kernels)
+        # hook(layer, stage, tensor) for named intermediates of every step; steps then run kernel by
+        # kernel, never from a recorded graph
+        self.debug_hook = None
         self.device = model.device
         self.arena = Arena(self.device)
         self.packer = StepPacker(cache.manager, len(cache.groups), cache.page_size)
@@ -225,6 +230,7 @@ class StepRunner:
                 raise StepError(f"request {e.rid!r}: only a single token can come from the sampled tokens")
 
         starts = {}
+        opened = []
         if reserved:
             for e in entries:               # the entry's tokens are the last positions that were reserved
                 starts[e.rid] = mgr.length(e.rid) + mgr.pending(e.rid) - len(e.tokens)
@@ -232,7 +238,6 @@ class StepRunner:
                     raise StepError(f"request {e.rid!r} brings {len(e.tokens)} tokens, {mgr.pending(e.rid)} are reserved")
         else:
             done = []
-            opened = []
             try:
                 for e in entries:
                     if e.rid not in mgr:
@@ -254,27 +259,42 @@ class StepRunner:
         order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
         n_decode = sum(1 for e in entries if len(e.tokens) == 1)
         graph_ok = (sample_records is not None and n_decode == len(entries) and self.use_graphs
+                    and self.debug_hook is None
                     and len(entries) <= self.max_graph_batch and all(list(e.want) == [0] for e in entries))
-        if graph_ok:
-            logits, ctx = self._run_graph(entries, starts, sample_records)
+        from ..kernels import ops
+        try:
+            with ops.kernel_mode_scope(self.kernels):
+                if graph_ok:
+                    logits, ctx = self._run_graph(entries, starts, sample_records)
+                else:
+                    logits, ctx = self._run_eager(entries, order, starts, sample_records)
+        except Exception:
+            # A launch that was refused (a size no kernel takes) leaves nothing half-done on the host:
+            # what this call reserved goes back, requests it opened are closed.  A caller that
+            # reserved itself decides what becomes of its requests.
             if not reserved:
                 for e in entries:
-                    mgr.commit(e.rid)
-            return logits, ctx
+                    mgr.rollback(e.rid)
+                for rid in opened:
+                    mgr.close(rid)
+            raise
+        if not reserved:                 # who reserves commits: the scheduler does it for its batches
+            for e in entries:
+                mgr.commit(e.rid)
+        return logits, ctx
 
+    def _run_eager(self, entries, order, starts, sample_records):
+        from ..kernels import ops
         offs, meta, n_words = self._layout(entries, order, pad_to=None, max_blocks=None, extra=sample_records)
         self._fill(self._staging_for(n_words), offs, meta, entries, order, starts, sample_records)
         dev = self._upload(n_words)
         ctx = self._context(dev, offs, meta, self.arena)
+        ctx.debug_hook = self.debug_hook
         self.last_ctx = ctx
         R = meta["R"]
         if any(e.from_sampled is not None for e in entries):
-            from ..kernels import ops
-            ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, cfg.vocab_size)
+            ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, self.model.config.vocab_size)
         logits = self.model.forward(ctx, ctx.want_rows if R else None, R)
-        if not reserved:                 # who reserves commits: the scheduler does it for its batches
-            for e in entries:
-                mgr.commit(e.rid)
         return logits, ctx
 
     def _context(self, dev, offs, meta, arena) -> StepContext:

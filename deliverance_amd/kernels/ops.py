@@ -65,7 +65,8 @@ def _check(rc: int):
 
 _VP, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 _ARGTYPES = {
-    "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _VP],
+    "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _F, _VP],
+    "da_copy_rows": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_take_tokens": [_VP, _VP, _VP, _I, _I, _I, _VP],
     "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
     "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
@@ -112,8 +113,8 @@ def _rows_2d(t: torch.Tensor, name: str):
 
 # ------------------------------------------------------------------------------- embedding
 def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
-          wpe: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
-    """out[n] = wte[tokens[n]] + wpe[positions[n]] in 32-bit."""
+          wpe: Optional[torch.Tensor], out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[n] = wte[tokens[n]] * scale + wpe[positions[n]] in 32-bit."""
     _dev(tokens, positions, wte, wpe, out)
     N, E = out.shape
     _need(tokens.dtype == torch.int32 and positions.dtype == torch.int32, "embed: ids must be int32")
@@ -123,8 +124,25 @@ def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
     if wpe is not None:
         _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: position table width differs from out")
     _check(_lib().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
-                                 _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, _stream()))
+                                 _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, float(scale), _stream()))
     return out
+
+
+def copy_rows(src: torch.Tensor, dst: torch.Tensor, rows: Optional[torch.Tensor] = None,
+              accumulate: bool = False) -> torch.Tensor:
+    """dst[r] (+)= src[rows[r]] (or src[r]); 32-bit and bfloat16 on either side, += into 32-bit."""
+    _dev(src, dst, rows)
+    _need(src.dim() == 2 and dst.dim() == 2 and src.is_contiguous() and dst.is_contiguous() and
+          src.shape[1] == dst.shape[1], "copy_rows: contiguous matrices of one width are needed")
+    R = dst.shape[0]
+    if rows is None:
+        _need(src.shape[0] >= R, "copy_rows: fewer source rows than destination rows")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= R, "copy_rows: rows must be int32 with a row each")
+    _need(not accumulate or dst.dtype == torch.float32, "copy_rows: accumulation needs a float32 destination")
+    _check(_lib().da_copy_rows(_ptr(src), _dt(src), _ptr(rows), _ptr(dst), _dt(dst), R, dst.shape[1],
+                               int(accumulate), _stream()))
+    return dst
 
 
 def take_tokens(tokens: torch.Tensor, src: torch.Tensor, sampled: torch.Tensor, vocab: int) -> torch.Tensor:
@@ -264,6 +282,26 @@ def set_kernel_mode(mode: str) -> None:
 
 def kernel_mode() -> str:
     return _MODE
+
+
+class kernel_mode_scope:
+    """The kernel mode of one engine while one of its steps is put on the device (two engines of
+    one process may differ)."""
+
+    def __init__(self, mode: str):
+        if mode not in ("tuned", "reference"):
+            raise ValueError("kernel mode must be 'tuned' or 'reference'")
+        self.mode = mode
+
+    def __enter__(self):
+        global _MODE
+        self._old, _MODE = _MODE, self.mode
+        return self
+
+    def __exit__(self, *exc):
+        global _MODE
+        _MODE = self._old
+        return False
 
 
 def _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, name):

@@ -80,21 +80,26 @@ class CausalLM:
     def _forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor], n_want: int) -> torch.Tensor:
         N = ctx.n_tokens
         x = ctx.buf("residual", N, self.config.width, torch.float32)
-        ops.embed(ctx.tokens, ctx.positions, self.token_table, self.embed_position.embed_table(), x)
+        ops.embed(ctx.tokens, ctx.positions, self.token_table, self.embed_position.embed_table(), x,
+                  self.config.embed_scale)
+        debug = ctx.debug_hook is not None          # the reference's stages: AbstractModel.java:1100,1107
+        if debug:
+            ctx.emit(-1, "input", x)
         for call in self.config.schedule:
             self.blocks[call.layer].forward(ctx, x, call)
+            if debug:
+                ctx.emit(call.layer, "layer_output", x)
         logits = ctx.buf("logits", n_want, self.config.vocab_size, torch.float32)
         if n_want == 0:
             return logits
-        from ..parts.norms import LayerNorm
-        if isinstance(self.final_norm, LayerNorm) and ops.can_fuse_ln(n_want, x, self.head_weight):
-            fn = self.final_norm                   # few wanted rows: norm and head in one kernel
-            return ops.linear_ln(x, want_rows, n_want, fn.weight, fn.bias, fn.eps, self.head_weight, None, logits)
+        ln = None if self.final_norm is None else self.final_norm.fusable_params()
+        if ln is not None and ops.can_fuse_ln(n_want, x, self.head_weight):
+            gain, bias, eps = ln                   # few wanted rows: norm and head in one kernel
+            return ops.linear_ln(x, want_rows, n_want, gain, bias, eps, self.head_weight, None, logits)
         if self.final_norm is not None:
             e = self.final_norm.forward(ctx, x, rows=want_rows, n_rows=n_want, out_name="final_norm")
         else:
-            e = ctx.buf("final_norm", n_want, self.config.width, ctx.dtype)
-            e.copy_(x.index_select(0, want_rows[:n_want].long()))
+            e = ops.copy_rows(x, ctx.buf("final_norm", n_want, self.config.width, ctx.dtype), rows=want_rows)
         ops.linear(e, self.head_weight, None, logits)
         return logits
 

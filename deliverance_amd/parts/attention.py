@@ -47,18 +47,18 @@ class CausalSelfAttention(Mixer):
 
     def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call) -> bool:
         """Small steps: LayerNorm, the q|k|v projection and the cache write in one kernel."""
-        from .norms import LayerNorm
         N = x.shape[0]
-        if not (isinstance(norm, LayerNorm) and self.position is None
-                and ops.can_fuse_ln(N, x, self.qkv_weight)):
+        ln = norm.fusable_params()
+        if ln is None or self.position is not None or not ops.can_fuse_ln(N, x, self.qkv_weight):
             return False
+        gain, bias, eps = ln
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
-        ops.linear_ln(x, None, N, norm.weight, norm.bias, norm.eps, self.qkv_weight, self.qkv_bias, qkv,
+        ops.linear_ln(x, None, N, gain, bias, eps, self.qkv_weight, self.qkv_bias, qkv,
                       kv_cache=slot if call.write else None, slot_map=ctx.slot_maps[group] if call.write else None,
                       q_cols=self.q_cols)
-        self._attend(ctx, qkv, x, slot, group)
+        self._attend(ctx, qkv, x, slot, group, call)
         return True
 
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
@@ -77,12 +77,18 @@ class CausalSelfAttention(Mixer):
             if call.write:
                 ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
                              self.n_kv_heads, self.head_dim)
-        self._attend(ctx, qkv, x, slot, group)
+        self._attend(ctx, qkv, x, slot, group, call)
 
-    def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int) -> None:
+    def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int,
+                call) -> None:
         N = qkv.shape[0]
         o = ctx.buf("attn_out", N, self.q_cols, ctx.dtype)
         ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
+        if ctx.debug_hook is not None:      # the reference's stage names (CausalSelfAttention.java:299-301,384)
+            ctx.emit(call.layer, "query_projection", qkv[:, :self.q_cols])
+            ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
+            ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:])
+            ctx.emit(call.layer, "attention_value", o)
         ops.linear(o, self.out_weight, self.out_bias, x, accumulate=True)
 
 

@@ -68,6 +68,9 @@ class StepContext:
         self.slot_maps: List[torch.Tensor] = []        # per group int32 [N]
         self.cache = None                              # engine.DeviceCache
         self._arena = None
+        # Called as hook(layer, stage, tensor) with copies of named intermediates (layer -1: the
+        # embedding), when set: core/src/main/java/io/teknek/deliverance/model/AbstractModel.java:122-128,505-515.
+        self.debug_hook: Optional[Callable] = None
 
     def buf(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         """A scratch matrix [rows, cols] that lives until the step ends."""
@@ -75,6 +78,11 @@ class StepContext:
 
     def group_of(self, cache_slot: int) -> int:
         return self.cache.group_of_slot[cache_slot]
+
+    def emit(self, layer: int, stage: str, tensor: torch.Tensor) -> None:
+        """Hand a named intermediate of this step to the debug hook, if there is one."""
+        if self.debug_hook is not None:
+            self.debug_hook(layer, stage, tensor.detach().clone())
 
 
 class Arena:
@@ -98,6 +106,11 @@ class Norm:
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
                 n_rows: Optional[int] = None, out_name: str = "norm") -> torch.Tensor:
         raise NotImplementedError
+
+    def fusable_params(self):
+        """(gain, bias or None, eps) when this norm is a LayerNorm that a product kernel can apply to
+        its own rows (``ops.linear_ln``); None when the norm must run as a kernel of its own."""
+        return None
 
 
 class Mixer:

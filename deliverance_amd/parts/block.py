@@ -1,11 +1,13 @@
 """The arrangement of one block: optional norms around a mixer and a feed-forward, each
 adding into the 32-bit residual stream.
 Reference: core/src/main/java/io/teknek/deliverance/generator/TransformerBlock.java:161-200
-(five optional norm places :26-32; GPT-2 uses the two pre-norms :35-41)."""
+(five optional norm places :26-32; GPT-2 uses the two pre-norms :35-41; a norm after a part acts
+on the part's output before the residual add :172-176,184-188)."""
 from __future__ import annotations
 
 import torch
 
+from ..kernels import ops
 from .base import StepContext, build_feed_forward, build_mixer, build_norm
 
 
@@ -21,26 +23,42 @@ class Block:
         self.mixer = build_mixer(spec.mixer, params["mixer"], dtype, device)
         self.feed_forward = None if spec.feed_forward is None else \
             build_feed_forward(spec.feed_forward, params["feed_forward"], dtype, device)
-        if self.post_mixer_norm is not None or self.post_ff_norm is not None:
-            # A norm after a part acts on the part's output before the residual add, which
-            # needs the part to write to a buffer of its own instead of into the stream.
-            raise NotImplementedError("post-part norms are not wired yet")
 
     @staticmethod
     def _normed(ctx, x, pre):
         if pre is not None:
             return pre.forward(ctx, x)
-        h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)
-        h.copy_(x)
-        return h
+        h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)      # no norm in front: the stream, converted
+        return ops.copy_rows(x, h)
+
+    @staticmethod
+    def _part(ctx, x, pre, post, run, run_normed):
+        """One part of the block.  Parts add into the tensor they are given.  Without a norm behind
+        the part that tensor is the residual stream; with one, the part adds into a zeroed buffer
+        of its own, whose norm is then added to the stream."""
+        target = x
+        if post is not None:
+            target = ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32)
+            target.zero_()
+        # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
+        # of it itself (fused into its first product) and returns True, or returns False to
+        # decline this step.  That needs the part's input and the tensor it adds into to be the same.
+        if not (post is None and pre is not None and run_normed is not None and run_normed(pre)):
+            run(Block._normed(ctx, x, pre), target)
+        if post is not None:
+            ops.copy_rows(post.forward(ctx, target, out_name="post_norm"), x, accumulate=True)
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
-        # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm itself
-        # (fused into its first product) and returns True, or returns False to decline this step.
         fused = getattr(self.mixer, "forward_normed", None)
-        if not (fused is not None and self.pre_mixer_norm is not None and fused(ctx, self.pre_mixer_norm, x, call)):
-            self.mixer.forward(ctx, self._normed(ctx, x, self.pre_mixer_norm), x, call)
+        self._part(ctx, x, self.pre_mixer_norm, self.post_mixer_norm,
+                   lambda h, into: self.mixer.forward(ctx, h, into, call),
+                   None if fused is None else (lambda norm: fused(ctx, norm, x, call)))
+        if ctx.debug_hook is not None:
+            ctx.emit(call.layer, "post_attention_residual", x)
         if self.feed_forward is not None:
             fused = getattr(self.feed_forward, "forward_normed", None)
-            if not (fused is not None and self.pre_ff_norm is not None and fused(ctx, self.pre_ff_norm, x)):
-                self.feed_forward.forward(ctx, self._normed(ctx, x, self.pre_ff_norm), x)
+            self._part(ctx, x, self.pre_ff_norm, self.post_ff_norm,
+                       lambda h, into: self.feed_forward.forward(ctx, h, into),
+                       None if fused is None else (lambda norm: fused(ctx, norm, x)))
+            if ctx.debug_hook is not None:
+                ctx.emit(call.layer, "post_ff_residual", x)

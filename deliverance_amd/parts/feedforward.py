@@ -27,13 +27,13 @@ class DenseFeedForward(FeedForward):
 
     def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor) -> bool:
         """Small steps: LayerNorm, fc, bias and activation in one kernel."""
-        from .norms import LayerNorm
         N = x.shape[0]
-        if not (isinstance(norm, LayerNorm) and ops.can_fuse_ln(N, x, self.fc_weight)):
+        ln = norm.fusable_params()
+        if ln is None or not ops.can_fuse_ln(N, x, self.fc_weight):
             return False
+        gain, bias, eps = ln
         mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)
-        ops.linear_ln(x, None, N, norm.weight, norm.bias, norm.eps, self.fc_weight, self.fc_bias, mid,
-                      act=self.activation)
+        ops.linear_ln(x, None, N, gain, bias, eps, self.fc_weight, self.fc_bias, mid, act=self.activation)
         ops.linear(mid, self.proj_weight, self.proj_bias, x, accumulate=True)
         return True
 

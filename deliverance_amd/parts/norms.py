@@ -25,5 +25,8 @@ class LayerNorm(Norm):
         out = ctx.buf(out_name, R, self.width, ctx.dtype)
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)
 
+    def fusable_params(self):
+        return self.weight, self.bias, self.eps
+
 
 register_norm("layernorm", LayerNorm)

@@ -64,5 +64,20 @@ def model_b(tmp_path_factory):
 
 
 @pytest.fixture(scope="session")
-def models(model_a, model_b):
-    return {"A": model_a, "B": model_b}
+def model_a32(tmp_path_factory):
+    """Configuration A stored in 32-bit, as openai-community/gpt2 ships."""
+    import helpers
+    return helpers.make_model(tmp_path_factory.mktemp("tiny_a32"), helpers.CONFIG_A, seed=2, store_dtype="float32")
+
+
+@pytest.fixture(scope="session")
+def model_b32(tmp_path_factory):
+    """Configuration B stored in 32-bit, with a head of its own (``tie_word_embeddings`` false)."""
+    import helpers
+    cfg = dict(helpers.CONFIG_B, tie_word_embeddings=False)
+    return helpers.make_model(tmp_path_factory.mktemp("tiny_b32"), cfg, seed=3, store_dtype="float32")
+
+
+@pytest.fixture(scope="session")
+def models(model_a, model_b, model_a32, model_b32):
+    return {"A": model_a, "B": model_b, "A32": model_a32, "B32": model_b32}

@@ -24,13 +24,16 @@ SIMT = os.environ.get("DELIVERANCE_SIMT") == "1"
 DEVICE = "cpu" if SIMT else "cuda:0"
 
 
-def trace_session(folder, dtype, max_tokens, page_size=16, poison_freed=False):
-    """The engine's trace session on the GPU, or its stand-in on the simulated kernels."""
+def trace_session(folder, dtype, max_tokens, page_size=16, poison_freed=False, **options):
+    """The engine's trace session on the GPU, or its stand-in on the simulated kernels (which has no
+    recorded graphs: ``use_graphs`` is dropped there)."""
     if SIMT:
         from simt import harness
-        return harness.SimTraceSession(None, str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed)
+        options.pop("use_graphs", None)
+        return harness.SimTraceSession(None, str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed,
+                                       **options)
     from deliverance_amd.trace import TraceSession
-    return TraceSession(str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed)
+    return TraceSession(str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed, **options)
 
 
 def skip_in_simulation_if(cond, why="too much arithmetic for the simulated kernels"):
@@ -39,8 +42,8 @@ def skip_in_simulation_if(cond, why="too much arithmetic for the simulated kerne
         pytest.skip(why)
 
 
-# Absolute tolerances on logits (their magnitude is about 1 on these models).
-ATOL = {"float32": 5e-6, "bfloat16": 1.5e-2}
+# Absolute tolerance on 32-bit logits (their magnitude is about 1 on these models).
+ATOL = {"float32": 5e-6}
 
 
 class TinyModel:
@@ -63,9 +66,13 @@ class TinyModel:
         return [int(t) for t in rng.integers(0, self.cfg["vocab_size"], size=length)]
 
 
-def make_model(folder, cfg, seed):
+def make_model(folder, cfg, seed, store_dtype="bfloat16"):
+    """A model folder with random weights, stored in bfloat16 or (as openai-community/gpt2 ships) in
+    32-bit: those weights are not bfloat16 numbers, so the 32-bit path meets them unrounded and the
+    bfloat16 path takes its kernels for 32-bit parameter vectors and tables."""
+    import torch
     from deliverance_amd.random_model import random_model
-    random_model(str(folder), cfg, seed)
+    random_model(str(folder), cfg, seed, {"bfloat16": torch.bfloat16, "float32": torch.float32}[store_dtype])
     return TinyModel(folder, cfg, seed)
 
 
@@ -155,14 +162,38 @@ def replay(session, steps):
     return {rid: np.stack(rows) for rid, rows in got.items()}
 
 
-def check_against_plain(model: TinyModel, got, requests, dtype, what=""):
-    atol = ATOL[dtype]
+# bfloat16 bounds relative to the logits' root mean square: the largest error and the rms error (about
+# four bfloat16 roundings of 2^-9 each end to end)
+BF16_MAX_OF_RMS, BF16_RMS_OF_RMS = 4e-2, 2.0 ** -7
+
+
+def bf16_token_slack(plain_row):
+    """How far below the plain maximum a token picked in bfloat16 may lie: two logits, each off by the
+    largest error the bfloat16 bound allows."""
+    return 2 * BF16_MAX_OF_RMS * float(np.sqrt((np.asarray(plain_row) ** 2).mean()))
+
+
+def check_against_plain(model: TinyModel, got, requests, dtype, what="", rows=None):
+    """32-bit: every logit within ATOL of the plain model's.  bfloat16: the largest error within 4 % of
+    the logits' rms and the rms error within 2^-7 of it, at every size (the logits' rms is 0.16 to 0.2 on
+    the tiny models and 0.55 to 0.8 at the benchmark models' layer sizes).  ``rows[rid]`` names the
+    positions that ``got[rid]`` holds when it does not hold all."""
     for rid, ids in requests:
         ref = model.plain_logits(ids)
+        if rows is not None:
+            ref = ref[rows[rid]]
         out = got[rid]
         assert out.shape == ref.shape, f"{what} {rid}: shape {out.shape} vs {ref.shape}"
         err = np.abs(out.astype(np.float64) - ref)
         worst = np.unravel_index(np.argmax(err), err.shape)
+        if dtype == "float32":
+            atol = ATOL[dtype]
+        else:
+            rms = float(np.sqrt((model.plain_logits(ids) ** 2).mean()))
+            atol = BF16_MAX_OF_RMS * rms
+            rms_err = float(np.sqrt((err ** 2).mean()))
+            assert rms_err <= BF16_RMS_OF_RMS * rms, (f"{what} request {rid} ({dtype}): rms error {rms_err:.3e} > "
+                                                      f"2^-7 of the logits' rms {rms:.3e}")
         assert err.max() <= atol, (f"{what} request {rid} ({dtype}): max abs error {err.max():.3e} > {atol:.1e}; "
                                    f"first bad position {int(np.argmax(err.max(axis=1) > atol))}, worst at "
                                    f"position {worst[0]} token {worst[1]}")

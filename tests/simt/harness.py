@@ -294,43 +294,39 @@ def make_runner(model, cache, sim: Sim = None):
     return r
 
 
-class SimTraceSession:
-    """What ``deliverance_amd.trace.TraceSession`` is on the GPU, on the simulated kernels.  With
-    ``sim`` the model's tensors, the cache and the scratch buffers live in guarded memory (use with
-    ``Sim.patched()``); without, they are ordinary CPU tensors (use with ``patched(auto_guard=True)``)."""
+def SimTraceSession(sim, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16,
+                    poison_freed: bool = False, **options):
+    """What ``deliverance_amd.trace.TraceSession`` is on the GPU, on the simulated kernels: the same
+    class with the step runner's host-to-device copy replaced.  With ``sim`` the model's tensors,
+    the cache and the scratch buffers live in guarded memory (use with ``Sim.patched()``); without,
+    they are ordinary CPU tensors (use with ``patched(auto_guard=True)``)."""
+    from deliverance_amd.trace import TraceSession
 
-    def __init__(self, sim, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16,
-                 poison_freed: bool = False):
-        from deliverance_amd import models  # noqa: F401
-        from deliverance_amd.engine.device_cache import DeviceCache
-        from deliverance_amd.models.causal_lm import load_model
-        tdtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
-        self.sim = sim
-        self.model = load_model(model_dir, tdtype, "cpu")
-        self.cache = DeviceCache(self.model.cache_needs(), tdtype, "cpu", page_size, max(max_tokens, 64),
-                                 n_state_slots=8, poison_freed=poison_freed)
-        if sim is not None:
-            sim.rehome(self.model, "model")
-            for g, t in enumerate(self.cache._group_tensors):
-                new = sim.like(t, f"cache group {g}")
-                self.cache._group_tensors[g] = new
-                for i, slot in enumerate(self.cache.groups[g].slots):
-                    self.cache.kv[slot] = new[i]
-            for slot, t in list(self.cache.state.items()):
-                self.cache.state[slot] = sim.like(t, f"state {slot}")
-        self.runner = make_runner(self.model, self.cache, sim)
+    class _Session(TraceSession):
+        def _make_runner(self, use_graphs, kernels):
+            if sim is not None:
+                sim.rehome(self.model, "model")
+                for g, t in enumerate(self.cache._group_tensors):
+                    new = sim.like(t, f"cache group {g}")
+                    self.cache._group_tensors[g] = new
+                    for i, slot in enumerate(self.cache.groups[g].slots):
+                        self.cache.kv[slot] = new[i]
+                for slot, t in list(self.cache.state.items()):
+                    self.cache.state[slot] = sim.like(t, f"state {slot}")
+            r = make_runner(self.model, self.cache, sim)
+            r.kernels = kernels
+            return r
 
-    def run_step(self, rec: dict):
-        from deliverance_amd.engine.step import StepEntry
-        entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
-        out = None
-        if entries:
-            logits, _ = self.runner.run(entries)
-            if logits.shape[0]:
-                out = logits.detach().to(torch.float32).contiguous().numpy().copy()
-        for rid in rec.get("end", []):
-            self.cache.manager.close(rid)
-        return out
+        def _drain(self):
+            pass
+
+        def run_step(self, rec):
+            out = super().run_step(rec)        # on the CPU this is a view of the step's logits buffer
+            return None if out is None else out.copy()
+
+    s = _Session(model_dir, dtype, max_tokens, page_size, device="cpu", poison_freed=poison_freed, **options)
+    s.sim = sim
+    return s
 
 
 def run_child(args, timeout: int = 900, env_extra=None):

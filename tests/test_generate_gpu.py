@@ -47,7 +47,7 @@ def test_greedy_in_bfloat16_stays_within_rounding_of_the_plain_maximum(models, n
             ids = list(prompt)
             for t in out.generated_tokens:
                 lg = m.plain_logits(ids)[-1]
-                assert lg[t] >= lg.max() - 2 * helpers.ATOL["bfloat16"]
+                assert lg[t] >= lg.max() - helpers.bf16_token_slack(lg)
                 ids.append(t)
 
 
@@ -175,7 +175,7 @@ def test_when_pages_run_out_requests_are_computed_again_with_the_same_result(mod
             ids = list(prompt)
             for t in out.generated_tokens:
                 lg = m.plain_logits(ids)[-1]
-                assert lg[t] >= lg.max() - 2 * helpers.ATOL["bfloat16"]
+                assert lg[t] >= lg.max() - helpers.bf16_token_slack(lg)
                 ids.append(t)
     tight.cache.manager.check()
     assert tight.cache.manager.pools[0].n_free == tight.cache.n_pages

@@ -22,11 +22,15 @@ def session_for(model, dtype, max_tokens, page_size=16):
 
 
 def requests_of(model, name):
-    return [(f"{name}{n}", model.prompt(n)) for n in LENGTHS[name]]
+    return [(f"{name}{n}", model.prompt(n)) for n in LENGTHS[name[0]]]
+
+
+# A, B: stored in bfloat16; A32, B32: stored in 32-bit (B32 with a head of its own)
+NAMES = ["A", "B", "A32", "B32"]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", NAMES)
 def test_whole(models, name, dtype):
     m = models[name]
     reqs = requests_of(m, name)
@@ -39,7 +43,7 @@ def test_whole(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", NAMES)
 def test_bulk_then_last_32_one_by_one(models, name, dtype):
     m = models[name]
     s = session_for(m, dtype, 128)
@@ -49,7 +53,7 @@ def test_bulk_then_last_32_one_by_one(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", NAMES)
 def test_portions_of_changing_size(models, name, dtype):
     m = models[name]
     s = session_for(m, dtype, 128)
@@ -60,10 +64,10 @@ def test_portions_of_changing_size(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", NAMES)
 def test_mixed_with_pages_used_again(models, name, dtype):
     m = models[name]
-    lengths = {"A": (40, 17, 56, 5, 33, 64, 23, 48), "B": (64, 9, 33, 88, 1, 50, 17, 40)}[name]
+    lengths = {"A": (40, 17, 56, 5, 33, 64, 23, 48), "B": (64, 9, 33, 88, 1, 50, 17, 40)}[name[0]]
     reqs = [(f"r{i}", m.prompt(n, salt=i)) for i, n in enumerate(lengths)]
     steps = helpers.trace_mixed(reqs, seed=3)
     assert max(len(s["entries"]) for s in steps) == 4
@@ -106,40 +110,43 @@ def test_long_decoding_and_first_tokens(model_a, dtype):
 
 BENCH_SIZES = {   # the layer sizes of the models that the benchmark runs, two layers of each
     "124m": dict(n_embd=768, n_head=12),
+    "355m": dict(n_embd=1024, n_head=16),       # the width at which the fused norm + product kernel ends
     "1.5b": dict(n_embd=1600, n_head=25),
 }
 
 
-@pytest.mark.parametrize("size", sorted(BENCH_SIZES))
-def test_layer_sizes_of_the_benchmark_models(size, tmp_path_factory):
-    """GPT-2 124M and 1.5B layer sizes (width, heads of 64, 4x inner width, the vocabulary of 50,257
-    that is no multiple of anything, 1,024 positions), two layers, against the plain model: one
-    request of 200 tokens (several key tiles, pages in any order) cut into portions and single
-    tokens beside a second request, in 32-bit and in bfloat16.
-
-    Logits here are four times those of the tiny models (rms 0.55 to 0.8 against 0.16 to 0.2), and
-    bfloat16 errors grow with them, so the bfloat16 bound is taken relative to the logits' rms: the
-    largest error below 4 % of it and the rms error below 2^-7 of it (four bfloat16 roundings).  On
-    the tiny models the absolute bound of the other tests is 7 to 9 % of the rms.  The 32-bit bound
-    is the absolute one of the other tests."""
+@pytest.fixture(scope="module", params=sorted(BENCH_SIZES))
+def bench_model(request, tmp_path_factory):
+    size = request.param
     cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, vocab_size=50257, n_positions=1024,
                layer_norm_epsilon=1e-5, activation_function="gelu_new", bos_token_id=50256, eos_token_id=50256,
                **BENCH_SIZES[size])
-    m = helpers.make_model(tmp_path_factory.mktemp("bench_" + size.replace(".", "_")), cfg, seed=5)
+    return helpers.make_model(tmp_path_factory.mktemp("bench_" + size.replace(".", "_")), cfg, seed=5)
+
+
+@pytest.mark.parametrize("mode", ["whole", "bulk+single", "portions", "mixed"])
+def test_layer_sizes_of_the_benchmark_models(bench_model, mode):
+    """GPT-2 124M, 355M and 1.5B layer sizes (width, heads of 64, 4x inner width, the vocabulary of
+    50,257 that is no multiple of anything, 1,024 positions), two layers, against the plain model, in
+    32-bit and in bfloat16, each way of cutting: a request of 200 tokens (several key tiles, pages in
+    any order) whole; most of it in one step and the last 32 tokens one by one; in portions of changing
+    size; and cut into portions and single tokens beside a second request."""
+    m = bench_model
+    helpers.skip_in_simulation_if(True)
     reqs = [("long", m.prompt(200)), ("short", m.prompt(75, salt=1))]
-    steps = helpers.trace_mixed(reqs, seed=3, max_live=2, prefill_sizes=(130, 2, 37, 64), decode_tail=6)
+    if mode == "whole":
+        steps = helpers.trace_whole(*reqs[0])
+    elif mode == "bulk+single":
+        steps = helpers.trace_bulk_then_single(*reqs[0], 32)
+    elif mode == "portions":
+        steps = helpers.trace_portions(*reqs[0], sizes=(67, 2, 33, 5, 16, 3))
+    else:
+        steps = helpers.trace_mixed(reqs, seed=3, max_live=2, prefill_sizes=(130, 2, 37, 64), decode_tail=6)
+    used = reqs if mode == "mixed" else reqs[:1]
     for dtype in DTYPES:
-        s = session_for(m, dtype, helpers.max_live_tokens(steps))
+        s = session_for(m, dtype, max(helpers.max_live_tokens(steps), 256))
         got = helpers.replay(s, steps)
-        if dtype == "float32":
-            helpers.check_against_plain(m, got, reqs, dtype, f"{size} sizes")
-        else:
-            for rid, ids in reqs:
-                ref = m.plain_logits(ids)
-                err = np.abs(got[rid].astype(np.float64) - ref)
-                rms = np.sqrt((ref ** 2).mean())
-                assert err.max() <= 4e-2 * rms, (rid, err.max(), rms, int(np.argmax(err.max(axis=1))))
-                assert np.sqrt((err ** 2).mean()) <= 2.0 ** -7 * rms
+        helpers.check_against_plain(m, got, used, dtype, f"{m.cfg['n_embd']} wide, {mode}")
         s.cache.manager.check()
 
 
