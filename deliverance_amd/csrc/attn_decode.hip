@@ -20,14 +20,21 @@
 
 #define DEC_MAX_D 256
 
+// Long contexts with few (sequence, head) pairs: the keys are also split over workgroups.  Workgroup
+// (pair, j) takes the keys j * span .. (j + 1) * span - 1 (span a multiple of 64) and leaves its
+// partial result (the weighted sum before the division, the maximum, the sum of weights: D + 2
+// floats) in a scratch buffer; a second kernel merges a pair's partial results in ascending order
+// of j.  The split depends on the step's shape only (pairs, widest block table), never on the
+// sequences' lengths, so a recorded graph can hold it.
+//
 // CPR: 16-byte pieces per key row, rounded up to a power of two (2..32)
-template <int CPR, int DEC_WAVES>
+template <int CPR, int DEC_WAVES, bool SPLIT>
 // (registers are held to 128 for head sizes up to 64, so that two workgroups share a compute unit)
 __global__ void __launch_bounds__(DEC_WAVES * DA_WAVE, (CPR <= 8 || DEC_WAVES == 16) ? 4 : 2)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                    const int* __restrict__ block_table, int max_blocks,
                    const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
-                   int window, bf16_t* __restrict__ out, int out_ld) {
+                   int window, bf16_t* __restrict__ out, int out_ld, int span, float* __restrict__ partial) {
   constexpr int G = DA_WAVE / CPR;            // keys scored side by side
   constexpr int DPL = CPR <= 8 ? 1 : CPR / 8; // value dimensions per lane: D <= 8 * CPR <= 64 * DPL
   __shared__ __attribute__((aligned(16))) float ps[DEC_WAVES][DA_WAVE];
@@ -51,7 +58,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   // starts with when nothing is cut off by a window (keys wave*64 ..).  Entries past the
   // sequence's pages are read (the table has max_blocks of them) and never used.
   const uint4 qraw = *(const uint4*)(q + (size_t)s * q_ld + h * D + (piece_ok ? piece * 8 : 0));
-  const int c0_guess = wave * DA_WAVE;
+  const int split0 = SPLIT ? (int)blockIdx.y * span : 0;          // the first key of this workgroup's share
+  const int c0_guess = split0 + wave * DA_WAVE;
   int btk0[CPR], btv0[8];
 #pragma unroll
   for (int i = 0; i < CPR; ++i) {
@@ -63,8 +71,11 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     const int pg = (c0_guess + g * 8) >> lg;
     btv0[g] = bt[pg < max_blocks ? pg : max_blocks - 1];
   }
-  const int p = seq_lens[s] - 1;                      // the row's position; it sees keys lo..p
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  // the row's position is seq_lens[s] - 1; it sees the keys lo..p (of which this workgroup takes its share)
+  const int p_row = seq_lens[s] - 1;
+  const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
+  const int p = SPLIT ? (p_row < split0 + span - 1 ? p_row : split0 + span - 1) : p_row;
+  const int lo = SPLIT ? (lo_row > split0 ? lo_row : split0) : lo_row;
 
   float acc[DPL];
 #pragma unroll
@@ -227,6 +238,18 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     f[w2] = part_m[w2] == -INFINITY ? 0.f : expf(part_m[w2] - mm);
     ll += part_l[w2] * f[w2];
   }
+  if (SPLIT) {
+    // the share's result before the division, its maximum and its sum of weights
+    float* mine = partial + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * (D + 2);
+    for (int d = t; d < D; d += DEC_WAVES * DA_WAVE) {
+      float o = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < DEC_WAVES; ++w2) o += part_acc[w2][d] * f[w2];
+      mine[d] = o;
+    }
+    if (t == 0) { mine[D] = mm; mine[D + 1] = ll; }
+    return;
+  }
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;     // a sequence of length 0 (padding) gives zeros
   for (int d = t; d < D; d += DEC_WAVES * DA_WAVE) {
     float o = 0.f;
@@ -236,9 +259,32 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   }
 }
 
-extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const int* block_table,
-                              int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
-                              float scale, int window, void* out, int out_ld, void* stream) {
+// The partial results of a (sequence, head) pair, merged in ascending order of the shares.
+__global__ void __launch_bounds__(256)
+attn_decode_merge_kernel(const float* __restrict__ partial, int n_splits, int Hq, int D,
+                         bf16_t* __restrict__ out, int out_ld) {
+  const int s = blockIdx.x / Hq, h = blockIdx.x % Hq;
+  const float* mine = partial + (size_t)blockIdx.x * n_splits * (D + 2);
+  float mm = -INFINITY;
+  for (int j = 0; j < n_splits; ++j) mm = fmaxf(mm, mine[(size_t)j * (D + 2) + D]);
+  float ll = 0.f;
+  for (int j = 0; j < n_splits; ++j) {
+    const float mj = mine[(size_t)j * (D + 2) + D];
+    ll += mine[(size_t)j * (D + 2) + D + 1] * (mj == -INFINITY ? 0.f : expf(mj - mm));
+  }
+  const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float o = 0.f;
+    for (int j = 0; j < n_splits; ++j) {
+      const float mj = mine[(size_t)j * (D + 2) + D];
+      o += mine[(size_t)j * (D + 2) + d] * (mj == -INFINITY ? 0.f : expf(mj - mm));
+    }
+    out[(size_t)s * out_ld + h * D + d] = f32_to_bf16(o * inv);
+  }
+}
+
+static int decode_checks(const void* q, int q_ld, const void* cache, int max_blocks, int S, int Hq, int Hkv, int D,
+                         int page, int window, int out_ld) {
   DA_REQUIRE(S >= 0 && Hq > 0 && Hkv > 0 && page > 0, "attn_decode: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_decode: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= DEC_MAX_D, "attn_decode: head size %d is not a multiple of 16 up to %d", D, DEC_MAX_D);
@@ -247,17 +293,25 @@ extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const 
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_decode: bad window or block table");
   DA_REQUIRE((uintptr_t)cache % 16 == 0 && (uintptr_t)q % 16 == 0 && q_ld % 8 == 0,
              "attn_decode: q and the cache must be 16-byte aligned");
-  if (S == 0) return 0;
+  return 0;
+}
+
+// n_splits == 1: one workgroup a (sequence, head) pair, no scratch.  n_splits > 1: the keys of a pair
+// go to n_splits workgroups of `span` keys each, partial results through `partial`
+// (S * Hq * n_splits * (D + 2) floats), then the merge kernel.
+static int decode_launch(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
+                         const int* seq_lens, int S, int Hq, int Hkv, int D, int page, float scale, int window,
+                         void* out, int out_ld, int n_splits, int span, float* partial, hipStream_t st) {
   const int pieces = D / 8;
   // 8 wavefronts; 16 where the workgroups are few (a context above 512 is then still one chunk a
   // wavefront, and the larger workgroup's start is paid once per compute unit)
-  const bool wide = (long)S * Hq <= 128 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
-  dim3 grid(S * Hq);
-  hipStream_t st = (hipStream_t)stream;
-#define LAUNCH2(C, W)                                                                                      \
-  hipLaunchKernelGGL((attn_decode_kernel<C, W>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld,   \
+  const bool wide = (long)S * Hq * n_splits <= 128 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
+  dim3 grid(S * Hq, n_splits);
+#define LAUNCH3(C, W, SP)                                                                                   \
+  hipLaunchKernelGGL((attn_decode_kernel<C, W, SP>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, \
                      (const bf16_t*)cache, block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, \
-                     (bf16_t*)out, out_ld)
+                     (bf16_t*)out, out_ld, span, partial)
+#define LAUNCH2(C, W) do { if (n_splits > 1) LAUNCH3(C, W, true); else LAUNCH3(C, W, false); } while (0)
 #define LAUNCH(C) do { if (wide) LAUNCH2(C, 16); else LAUNCH2(C, 8); } while (0)
   if (pieces <= 2) LAUNCH(2);
   else if (pieces <= 4) LAUNCH(4);
@@ -266,6 +320,50 @@ extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const 
   else LAUNCH(32);
 #undef LAUNCH
 #undef LAUNCH2
+#undef LAUNCH3
+  if (n_splits > 1)
+    hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(S * Hq), dim3(D <= 64 ? 64 : (D <= 128 ? 128 : 256)), 0, st,
+                       partial, n_splits, Hq, D, (bf16_t*)out, out_ld);
+  return 0;
+}
+
+extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const int* block_table,
+                              int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
+                              float scale, int window, void* out, int out_ld, void* stream) {
+  if (decode_checks(q, q_ld, cache, max_blocks, S, Hq, Hkv, D, page, window, out_ld)) return 1;
+  if (S == 0) return 0;
+  decode_launch(q, q_ld, cache, block_table, max_blocks, seq_lens, S, Hq, Hkv, D, page, scale, window, out, out_ld,
+                1, 0, nullptr, (hipStream_t)stream);
   DA_CHECK_LAUNCH("attn_decode");
+  return 0;
+}
+
+// The keys of every (sequence, head) pair split over n_splits workgroups; `workspace` holds the
+// partial results (da_attn_decode_split_bytes of it, 16-byte aligned).
+extern "C" long da_attn_decode_split_bytes(int S, int Hq, int D, int n_splits) {
+  return (long)S * Hq * n_splits * (D + 2) * (long)sizeof(float);
+}
+
+static int split_checks(int max_blocks, int page, int n_splits, int* span) {
+  DA_REQUIRE(n_splits >= 2 && n_splits <= 64, "attn_decode_split: %d shares (2 to 64 are taken)", n_splits);
+  const long keys = (long)max_blocks * page;
+  *span = (int)(((keys + n_splits - 1) / n_splits + DA_WAVE - 1) / DA_WAVE * DA_WAVE);
+  return 0;
+}
+
+extern "C" int da_attn_decode_split(const void* q, int q_ld, const void* cache, const int* block_table,
+                                    int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
+                                    float scale, int window, void* out, int out_ld, int n_splits, void* workspace,
+                                    long workspace_bytes, void* stream) {
+  if (decode_checks(q, q_ld, cache, max_blocks, S, Hq, Hkv, D, page, window, out_ld)) return 1;
+  int span = 0;
+  if (split_checks(max_blocks, page, n_splits, &span)) return 1;
+  DA_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= da_attn_decode_split_bytes(S, Hq, D, n_splits),
+             "attn_decode_split: the workspace holds %ld bytes, %ld are needed", workspace_bytes,
+             da_attn_decode_split_bytes(S, Hq, D, n_splits));
+  if (S == 0) return 0;
+  decode_launch(q, q_ld, cache, block_table, max_blocks, seq_lens, S, Hq, Hkv, D, page, scale, window, out, out_ld,
+                n_splits, span, (float*)workspace, (hipStream_t)stream);
+  DA_CHECK_LAUNCH("attn_decode_split");
   return 0;
 }

@@ -76,6 +76,7 @@ _ARGTYPES = {
     "da_kv_write": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_attn_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
     "da_attn_decode": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_decode_split": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
     "da_attn_prefill": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
     "da_sample": [_VP, _I, _I, _I, _VP, _VP, _VP],
     "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
@@ -431,19 +432,52 @@ def _attn_common(q, cache_slot, block_table, n_heads, out, name):
     return Hkv, page, D
 
 
+# Decode attention splits a (sequence, head) pair's keys over workgroups when the pairs alone leave most
+# of the chip idle and the context is long: shares of at least DECODE_SPLIT_MIN_KEYS keys, as many as
+# bring the workgroups to about DECODE_SPLIT_WORKGROUPS.  The choice reads the step's shape only (pairs
+# and the width of the block table), so that a recorded step keeps it.
+DECODE_SPLIT_MIN_KEYS = 1024
+DECODE_SPLIT_WORKGROUPS = 512
+DECODE_SPLIT_MAX = 32
+
+
+def decode_splits(n_seqs: int, n_heads: int, max_blocks: int, page: int) -> int:
+    by_keys = (max_blocks * page) // DECODE_SPLIT_MIN_KEYS
+    by_fill = DECODE_SPLIT_WORKGROUPS // max(1, n_seqs * n_heads)
+    n = min(by_keys, by_fill, DECODE_SPLIT_MAX)
+    return n if n >= 2 else 1
+
+
 def attention_decode(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
                      seq_lens: torch.Tensor, n_seqs: int, n_heads: int, scale: float,
-                     window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+                     window: Optional[int], out: torch.Tensor, n_splits: int = 1,
+                     workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One query row per sequence: row s of q belongs to sequence s and sits at position
-    seq_lens[s] - 1."""
+    seq_lens[s] - 1.  With ``n_splits`` > 1 every (sequence, head) pair's keys are shared out over
+    that many workgroups, whose partial results pass through ``workspace`` (float32,
+    ``decode_workspace_floats`` elements)."""
     Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_decode")
     _need(q.shape[0] >= n_seqs and out.shape[0] >= n_seqs and block_table.shape[0] >= n_seqs,
           "attention_decode: fewer rows than sequences")
     _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= n_seqs, "attention_decode: seq_lens must be int32 [S]")
-    _check(_lib().da_attn_decode(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+    if n_splits <= 1:
+        _check(_lib().da_attn_decode(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
+                                     block_table.shape[1], _ptr(seq_lens), n_seqs, n_heads, Hkv, D, page,
+                                     scale, int(window or 0), _ptr(out), out.stride(0), _stream()))
+        return out
+    need = decode_workspace_floats(n_seqs, n_heads, D, n_splits)
+    _need(workspace is not None and workspace.dtype == torch.float32 and workspace.is_contiguous()
+          and workspace.numel() >= need, f"attention_decode: the workspace must hold {need} float32")
+    _dev(workspace)
+    _check(_lib().da_attn_decode_split(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
                                        block_table.shape[1], _ptr(seq_lens), n_seqs, n_heads, Hkv, D, page,
-                                       scale, int(window or 0), _ptr(out), out.stride(0), _stream()))
+                                       scale, int(window or 0), _ptr(out), out.stride(0), n_splits,
+                                       _ptr(workspace), workspace.numel() * 4, _stream()))
     return out
+
+
+def decode_workspace_floats(n_seqs: int, n_heads: int, head_dim: int, n_splits: int) -> int:
+    return n_seqs * n_heads * n_splits * (head_dim + 2)
 
 
 def attention_prefill(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
@@ -473,7 +507,12 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
     if _MODE == "tuned" and q.dtype == torch.bfloat16:
         nd = ctx.n_decode
         if nd:
-            attention_decode(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, out)
+            page, D = cache_slot.shape[3], cache_slot.shape[4]
+            n_splits = decode_splits(nd, n_heads, bt.shape[1], page)
+            ws = None
+            if n_splits > 1:
+                ws = ctx.buf("decode_partial", 1, decode_workspace_floats(nd, n_heads, D, n_splits), torch.float32)
+            attention_decode(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, out, n_splits, ws)
         if ctx.n_seqs > nd:
             attention_prefill(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
                               ctx.max_query_len, n_heads, scale, window, out)

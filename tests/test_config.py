@@ -94,3 +94,11 @@ def test_engine_config_checks():
         EngineConfig(dtype="fp8")
     with pytest.raises(ValueError):
         EngineConfig(page_size=24)
+    # only the page sizes that every attention kernel takes: refused here, not at the first launch
+    for bad in (8, 48, 80, 128, 0, -16):
+        with pytest.raises(ValueError, match="page_size must be one of"):
+            EngineConfig(page_size=bad)
+    assert [EngineConfig(page_size=p).page_size for p in (16, 32, 64)] == [16, 32, 64]
+    assert EngineConfig().kernels == "tuned" and EngineConfig(kernels="reference").kernels == "reference"
+    with pytest.raises(ValueError, match="kernels must be one of"):
+        EngineConfig(kernels="fast")

@@ -215,3 +215,28 @@ def test_named_intermediates_of_a_step(models, dtype):
         assert np.abs(seen[(layer, "post_ff_residual")] - x).max() < tol, layer
         assert np.abs(seen[(layer, "layer_output")] - x).max() < tol, layer
     assert len(seen) == 1 + 7 * cfg["n_layer"]
+
+
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+    """2,304 positions: decode attention shares a sequence's keys out over two workgroups a head."""
+    cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=128, n_head=2, vocab_size=300,
+               n_positions=2304, layer_norm_epsilon=1e-5, activation_function="gelu_new", bos_token_id=0, eos_token_id=1)
+    return helpers.make_model(tmp_path_factory.mktemp("long"), cfg, seed=9)
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_decoding_over_a_long_context(long_model, graphs):
+    """A context of 2,200 tokens and one of 1,100 beside it, the last 24 tokens one by one: the decode
+    kernel splits the keys over workgroups (the block table spans more than 2,048 keys) and merges."""
+    from deliverance_amd.kernels import ops
+    m = long_model
+    helpers.skip_in_simulation_if(True)
+    reqs = [("far", m.prompt(2200, salt=1)), ("near", m.prompt(1100, salt=2))]
+    steps = decode_trace(reqs, [24, 24])
+    assert ops.decode_splits(2, 2, -(-2200 // 16), 16) == 2
+    s = helpers.trace_session(m.folder, "bfloat16", 4096, poison_freed=True, use_graphs=graphs, sample=graphs)
+    got = helpers.replay(s, steps)
+    helpers.check_against_plain(m, got, reqs, "bfloat16", f"long context, graphs={graphs}")
+    if graphs:
+        assert s.runner._graphs

@@ -42,6 +42,32 @@ def test_embed(ops, table_dtype):
     assert torch.equal(out, wte.float()[tok.long()])
 
 
+def test_embed_scale_and_row_copies(ops):
+    g = torch.Generator().manual_seed(2)
+    V, Pn, E, N = 300, 50, 72, 21
+    wte, wpe = bf(torch.randn(V, E, generator=g)).to(DEV), bf(torch.randn(Pn, E, generator=g)).to(DEV)
+    tok = torch.randint(0, V, (N,), generator=g, dtype=torch.int32).to(DEV)
+    pos = torch.randint(0, Pn, (N,), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.empty(N, E, device=DEV)
+    ops.embed(tok, pos, wte, wpe, out, scale=8.5)
+    assert torch.equal(out, wte.float()[tok.long()] * 8.5 + wpe.float()[pos.long()])
+    # rows gathered and converted; rows added into the 32-bit stream
+    rows = torch.tensor([20, 0, 7, 7, 3], dtype=torch.int32, device=DEV)
+    for dt in (torch.float32, torch.bfloat16):
+        dst = torch.empty(5, E, device=DEV, dtype=dt)
+        ops.copy_rows(out, dst, rows=rows)
+        assert torch.equal(dst, out[rows.long()].to(dt))
+        dst = torch.empty(N, E, device=DEV, dtype=dt)
+        ops.copy_rows(out, dst)
+        assert torch.equal(dst, out.to(dt))
+    acc = torch.randn(N, E, generator=g).to(DEV)
+    want = acc + bf(out).float()
+    ops.copy_rows(bf(out), acc, accumulate=True)
+    assert torch.equal(acc, want)
+    with pytest.raises(ops.KernelError, match="float32 destination"):
+        ops.copy_rows(out, bf(out), accumulate=True)
+
+
 @pytest.mark.parametrize("E,eps", [(7, 1e-5), (200, 1e-6), (1600, 1e-5), (64, 1e-1)])
 def test_layernorm(ops, E, eps):
     g = torch.Generator().manual_seed(1)
@@ -235,6 +261,40 @@ def test_attention_decode_kernel(ops, Hq, Hkv, D, page, window):
     assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("n_splits", [2, 3, 7, 16])
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(2, 2, 64, 16, None), (4, 2, 48, 32, None), (1, 1, 128, 64, 700),
+                                                  (3, 3, 16, 16, 90)])
+def test_attention_decode_with_keys_split_over_workgroups(ops, Hq, Hkv, D, page, window, n_splits):
+    """Every (sequence, head) pair's keys in ``n_splits`` shares with a merge in a fixed order: shares
+    that hold nothing (short sequences, a window that has passed them), one key, a share's first and
+    last key, sequences that end at a share's edge."""
+    width = 2100                                                   # keys the block table spans
+    span = -(-(-(-width // page) * page) // n_splits // 64) * 64    # what the kernel gives a share
+    lens = [1, 2, 63, span, span + 1, 2 * span - 1 if 2 * span - 1 <= width else width, 1030, width, 700]
+    case = PagedCase(lens=lens, new=[1] * len(lens), Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + n_splits)
+    assert case.bt.shape[1] == -(-width // page)
+    scale = 0.7 / math.sqrt(D)
+    out = torch.full_like(case.qcat, float("nan"))
+    ws = torch.full((ops.decode_workspace_floats(len(lens), Hq, D, n_splits),), float("nan"), device=DEV)
+    ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, out, n_splits, ws)
+    got = out.double().cpu().numpy()
+    assert np.isfinite(got).all()
+    assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
+    one = torch.empty_like(case.qcat)
+    ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, one)
+    assert (out.float() - one.float()).abs().max() < 2e-2          # the two kernels differ by rounding only
+    with pytest.raises(ops.KernelError, match="workspace"):
+        ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, out, n_splits, ws[:10])
+
+
+def test_when_decode_attention_splits_its_keys(ops):
+    assert ops.decode_splits(1, 12, 64, 16) == 1                   # 1,024 keys: one share
+    assert ops.decode_splits(1, 12, 256, 16) == 4                  # 4,096 keys, 12 pairs: shares of 1,024
+    assert ops.decode_splits(8, 25, 256, 16) == 2                  # 200 pairs: two shares fill the chip
+    assert ops.decode_splits(64, 12, 256, 16) == 1                 # 768 pairs fill it alone
+    assert ops.decode_splits(1, 1, 4096, 16) == 32                 # never more than 32
+
+
 @pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
                                                   (3, 3, 128, 64, None), (12, 12, 64, 16, None), (5, 5, 64, 16, 100),
                                                   (2, 2, 256, 16, None), (2, 2, 240, 16, None), (3, 1, 64, 32, 200)])
@@ -249,6 +309,29 @@ def test_attention_prefill_kernel(ops, Hq, Hkv, D, page, window):
     got = out.double().cpu().numpy()
     assert np.isfinite(got).all()
     assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_row_that_sees_no_key_gives_zeros(ops, dtype):
+    """The padding rows of a fixed-shape decode step: length 0, a block table of -1.  Zeros, never NaN
+    (NaN would spread through the row's residual into its logits and into the sampling kernel)."""
+    Hq, Hkv, D, page = 4, 2, 32, 16
+    case = PagedCase(lens=[20, 7], new=[1, 1], Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=dtype, seed=8)
+    q = torch.cat([case.qcat, torch.randn(2, Hq * D).to(dtype).to(DEV)])
+    bt = torch.cat([case.bt, torch.full((2, case.bt.shape[1]), -1, dtype=torch.int32, device=DEV)])
+    seq_of = torch.tensor([0, 1, 2, 3], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([19, 6, 0, 0], dtype=torch.int32, device=DEV)
+    out = torch.full_like(q, float("nan"))
+    ops.attention_ref(q, case.cache, bt, seq_of, pos, Hq, 0.2, None, out)
+    want = case.plain(0.2, None)
+    assert np.abs(out[:2].double().cpu().numpy() - want).max() < ATT_TOL[dtype]
+    assert torch.equal(out[2:], torch.zeros_like(out[2:]))
+    if dtype == torch.bfloat16:
+        out2 = torch.full_like(q, float("nan"))
+        lens = torch.tensor([20, 7, 0, 0], dtype=torch.int32, device=DEV)
+        ops.attention_decode(q, case.cache, bt, lens, 4, Hq, 0.2, None, out2)
+        assert torch.equal(out2[2:], torch.zeros_like(out2[2:]))
+        assert np.abs(out2[:2].double().cpu().numpy() - want).max() < ATT_TOL[dtype]
 
 
 def test_attention_reference_vector_shape(ops):

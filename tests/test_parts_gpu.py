@@ -195,3 +195,52 @@ def test_block_part_and_fused_small_steps(model_b, dtype):
         blk.forward(ctx, x, LayerCall(layer, 0, True))
         want = P.block(x0.double().numpy(), model_b.W, layer, model_b.plain_cfg)
         assert np.abs(x.double().cpu().numpy() - want).max() < TOL[dtype] * 2, T
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("pre", [True, False])
+def test_block_with_norms_behind_its_parts(model_b, dtype, pre):
+    """The block's other norm places (TransformerBlock.java:26-32,172-176,184-188): a norm behind a
+    part acts on the part's output before it joins the stream,
+        x1 = x + N_post(Attn(N_pre(x)));  x2 = x1 + N_post'(MLP(N_pre'(x1))),
+    with or without the norms in front (without: the part reads the stream itself)."""
+    import dataclasses
+    from deliverance_amd.config import Gpt2Config, LayerCall
+    from deliverance_amd.models import gpt2 as arch
+    from deliverance_amd.parts import Block
+    from deliverance_amd.weights import load_declared
+    mc = Gpt2Config.from_dict(helpers.CONFIG_B).to_model_config()
+    bound = arch.bind_tensors(mc, load_declared(model_b.folder, arch.declare_tensors(mc)))
+    layer, W, cfg = 1, model_b.W, model_b.plain_cfg
+    spec = mc.layers[layer]
+    norm = spec.pre_mixer_norm
+    spec = dataclasses.replace(spec, post_mixer_norm=norm, post_ff_norm=norm,
+                               pre_mixer_norm=norm if pre else None, pre_ff_norm=norm if pre else None)
+    params = dict(bound["layers"][layer])
+    # the norms behind the parts borrow the other layers' parameters
+    post = {"post_mixer_norm": ("h.0.ln_1", "h.0.ln_1"), "post_ff_norm": ("h.2.ln_2", "h.2.ln_2")}
+    for key, (wn, bn) in post.items():
+        params[key] = {"weight": torch.from_numpy(W[wn + ".weight"]).to(torch.bfloat16),
+                       "bias": torch.from_numpy(W[bn + ".bias"]).to(torch.bfloat16)}
+    blk = Block(spec, params, dtype, DEV)
+    eps = cfg["layer_norm_epsilon"]
+    H, E = cfg["n_head"], cfg["n_embd"]
+    scale = 1.0 / math.sqrt(E // H) / (layer + 1)          # config B scales by the layer's number
+    g = torch.Generator().manual_seed(6)
+    for T in (40, 5):
+        x0 = torch.randn(T, E, generator=g)
+        ctx = make_ctx(dtype, [T], [0], 2, 48)
+        x = x0.clone().to(DEV)
+        blk.forward(ctx, x, LayerCall(layer, 0, True))
+        xn = x0.double().numpy()
+        a = P.layer_norm(xn, W[f"h.{layer}.ln_1.weight"], W[f"h.{layer}.ln_1.bias"], eps) if pre else xn
+        o = P.attention_block(a, W, layer, H, scale)
+        x1 = xn + P.layer_norm(o, W["h.0.ln_1.weight"], W["h.0.ln_1.bias"], eps)
+        mm = P.layer_norm(x1, W[f"h.{layer}.ln_2.weight"], W[f"h.{layer}.ln_2.bias"], eps) if pre else x1
+        f = P.mlp_block(mm, W, layer, cfg["activation_function"])
+        want = x1 + P.layer_norm(f, W["h.2.ln_2.weight"], W["h.2.ln_2.bias"], eps)
+        # a norm amplifies its input's rounding: parts' outputs are small (weights of 0.02), normalised to 1
+        tol = {torch.float32: 2e-4, torch.bfloat16: 1.5e-1}[dtype]
+        assert np.abs(x.double().cpu().numpy() - want).max() < tol, (T, pre)
+        wrong = xn + o + f                                   # (a block that forgot the norms is far off)
+        assert np.abs(want - wrong).max() > 1.0

@@ -61,3 +61,23 @@ def test_records_draw_in_the_reference_order():
     f = fields(GeneratorParameters(temperature=0.8, xtc_threshold=0.1, xtc_probability=0.5), r)
     ref.next_float(); ref.next_float(); d = ref.next_float()
     assert f[5] == pytest.approx(0.1) and f[6] == int(not d > 0.5) and r.next_float() == ref.next_float()
+
+
+def test_the_reference_default_nucleus_is_an_explicit_option_here():
+    """The reference sets top_p = 0.10 when the temperature is positive and no filter is given
+    (core/src/main/java/io/teknek/deliverance/model/AbstractGeneratorSampler.java:107-110); here no
+    filter means none.  On the reference's own test logits (TopKSamplerTest.java:23-54: 5, 4, 3, 2, 1;
+    softmax 0.636, 0.234, 0.086, 0.032, 0.012) a nucleus of 0.10 holds the first token alone, so with
+    ``top_p=0.1`` every draw gives token 0, as the reference's default does; without a filter the draw
+    walks the whole softmax."""
+    import numpy as np
+    logits = np.array([5.0, 4.0, 3.0, 2.0, 1.0])
+    cdf = np.cumsum(np.exp(logits - 5.0) / np.exp(logits - 5.0).sum())
+    for u in (0.0, 0.3, 0.64, 0.9, 0.999999):
+        assert P.sample_top_k_top_p(logits, 1.0, None, 0.10, None, u) == 0
+        assert P.sample_top_k_top_p(logits, 1.0, None, None, None, u) == int(np.searchsorted(cdf, u, side="right"))
+    # the record that goes to the device carries exactly what was asked for: no silent nucleus
+    fields = struct.unpack("<fififfii", device_record(GeneratorParameters(temperature=1.0), JavaRandom(1), 5))
+    assert fields[1] == 0 and fields[2] == 0.0
+    fields = struct.unpack("<fififfii", device_record(GeneratorParameters(temperature=1.0, top_p=0.1), JavaRandom(1), 5))
+    assert fields[2] == pytest.approx(0.1)

@@ -108,3 +108,32 @@ def test_a_single_token_may_come_from_the_step_before():
     mgr.open("a"); mgr.extend("a", 5); mgr.commit("a")
     order, starts, meta, v = pack(packer, mgr, [StepEntry("a", [0], [0], from_sampled=3), StepEntry("b", [4, 5, 6], [2])])
     assert v["token_src"].tolist() == [3, -1, -1, -1] and v["positions"].tolist() == [5, 0, 1, 2]
+
+
+def test_a_launch_that_fails_leaves_no_reservation_behind(tmp_path):
+    """The step function reserves positions, then launches.  When the launch is refused (here: the
+    kernels are asked to run on CPU tensors, which they refuse) the reservation goes back and the
+    requests that the call opened are closed; a request that was open before keeps what it had."""
+    import torch
+    import helpers
+    from deliverance_amd.engine.device_cache import DeviceCache
+    from deliverance_amd.engine.step import StepEntry
+    from deliverance_amd.kernels import ops
+    from deliverance_amd.models.causal_lm import load_model
+    from simt import harness
+    m = helpers.make_model(tmp_path, helpers.CONFIG_A, 0)
+    model = load_model(m.folder, torch.float32, "cpu")
+    with pytest.raises(ValueError, match="page_size must be one of"):
+        DeviceCache(model.cache_needs(), torch.float32, "cpu", 48, 256, n_state_slots=4)
+    cache = DeviceCache(model.cache_needs(), torch.float32, "cpu", 16, 256, n_state_slots=4)
+    runner = harness.make_runner(model, cache)          # the step function without pinned memory
+    mgr = cache.manager
+    mgr.open("old")
+    mgr.extend("old", 20)
+    mgr.commit("old")
+    free = mgr.pools[0].n_free
+    with pytest.raises((ops.KernelError, RuntimeError)):       # no GPU here: the first launch refuses
+        runner.run([StepEntry("old", [1] * 30, [29]), StepEntry("new", [2] * 40, [])])
+    assert mgr.live() == ["old"] and mgr.length("old") == 20 and mgr.pending("old") == 0
+    assert mgr.pools[0].n_free == free
+    mgr.check()
