@@ -367,3 +367,54 @@ extern "C" int da_attn_decode_split(const void* q, int q_ld, const void* cache, 
   DA_CHECK_LAUNCH("attn_decode_split");
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same without a workspace argument and without any allocation (see no_alloc.h).
+// ---------------------------------------------------------------------------------------------
+#include "no_alloc.h"
+#include <mutex>
+
+static __device__ __align__(256) unsigned char scratch[DA_DECODE_STATIC_SCRATCH_BYTES];
+
+#define DA_MAX_DEVICES 64
+static void* g_scratch_of_device[DA_MAX_DEVICES];      // the array's address on each GPU, asked for once
+static std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the current device.  In host code the array's name is only a handle
+// for the runtime; the memory's address differs from GPU to GPU and comes from hipGetSymbolAddress.
+static int static_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  DA_REQUIRE(e == hipSuccess && dev >= 0 && dev < DA_MAX_DEVICES, "attn_decode_split_static: no current device (%s)",
+             hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_of_device[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    DA_REQUIRE(e == hipSuccess && p, "attn_decode_split_static: the scratch buffer's address is not known (%s)",
+               hipGetErrorString(e));
+    g_scratch_of_device[dev] = p;
+  }
+  *ptr = (float*)g_scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" int da_attn_decode_split_static(const void* q, int q_ld, const void* cache, const int* block_table,
+                                           int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D,
+                                           int page, float scale, int window, void* out, int out_ld, int n_splits,
+                                           void* stream) {
+  if (decode_checks(q, q_ld, cache, max_blocks, S, Hq, Hkv, D, page, window, out_ld)) return 1;
+  int span = 0;
+  if (split_checks(max_blocks, page, n_splits, &span)) return 1;
+  const long need = da_attn_decode_split_bytes(S, Hq, D, n_splits);
+  DA_REQUIRE(need <= (long)DA_DECODE_STATIC_SCRATCH_BYTES,
+             "attn_decode_split_static: %d sequences x %d heads x %d shares of head size %d need %ld bytes of scratch, "
+             "the library holds %ld", S, Hq, n_splits, D, need, (long)DA_DECODE_STATIC_SCRATCH_BYTES);
+  if (S == 0) return 0;
+  float* partial = nullptr;
+  if (static_scratch(&partial)) return 1;
+  decode_launch(q, q_ld, cache, block_table, max_blocks, seq_lens, S, Hq, Hkv, D, page, scale, window, out, out_ld,
+                n_splits, span, partial, (hipStream_t)stream);
+  DA_CHECK_LAUNCH("attn_decode_split_static");
+  return 0;
+}

@@ -47,6 +47,11 @@ typedef void* hipStream_t;
 typedef int hipError_t;
 #define hipSuccess 0
 static inline hipError_t hipGetLastError() { return hipSuccess; }
+static inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
+#define __align__(n) __attribute__((aligned(n)))
+#define HIP_SYMBOL(x) (x)
+template <class T>
+static inline hipError_t hipGetSymbolAddress(void** ptr, T& symbol) { *ptr = (void*)&symbol; return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "no error"; }
 
 namespace simt {
