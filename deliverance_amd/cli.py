@@ -36,7 +36,7 @@ def _ids(s: str):
 
 def cmd_generate(a) -> int:
     from . import AutoModelForCausalLM, EngineConfig, GeneratorParameters
-    from .profiler import InferenceProfiler
+    from .profiler import InferenceProfiler, KernelProfiler
     prompts = [_ids(p) for p in (a.prompt_ids or [])]
     if a.suite_file:
         with open(a.suite_file) as f:
@@ -58,6 +58,7 @@ def cmd_generate(a) -> int:
                                       max_cached_tokens=a.max_cached_tokens).items() if v is not None})
     if a.profile_stages:
         InferenceProfiler.enable(sync=True)
+        KernelProfiler.enable()            # every kernel launch timed on the device (no recorded graphs meanwhile)
     model = AutoModelForCausalLM.from_pretrained(a.model, engine_config=EngineConfig(**cfg))
     params = GeneratorParameters(temperature=a.temperature, seed=a.seed, max_tokens=a.max_tokens, ntokens=a.ntokens,
                                  top_k=a.top_k, top_p=a.top_p, uniform_top_p=a.uniform_top_p,
@@ -66,6 +67,7 @@ def cmd_generate(a) -> int:
     for p in prompts[:a.warmup_cases]:
         model.generate(p, params)
     InferenceProfiler.reset()
+    KernelProfiler.reset()
     t0 = time.perf_counter()
     outs = model.generate(prompts, params) if a.batch else [model.generate(p, params) for p in prompts]
     wall = time.perf_counter() - t0
@@ -97,6 +99,8 @@ def cmd_generate(a) -> int:
                 f.write(json.dumps(r) + "\n")
     if a.profile_stages:
         print(InferenceProfiler.summary("(stages drained at their end)"), file=sys.stderr)
+        print(KernelProfiler.summary("(device time per kernel against what it must move and compute; % of 8 TB/s or of "
+                                     "the matrix peak, whichever binds)"), file=sys.stderr)
     return 0
 
 

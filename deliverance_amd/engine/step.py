@@ -258,8 +258,9 @@ class StepRunner:
         # one-token entries first (the decode kernels take them), portions after
         order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
         n_decode = sum(1 for e in entries if len(e.tokens) == 1)
+        from ..profiler import KernelProfiler
         graph_ok = (sample_records is not None and n_decode == len(entries) and self.use_graphs
-                    and self.debug_hook is None
+                    and self.debug_hook is None and not KernelProfiler.enabled
                     and len(entries) <= self.max_graph_batch and all(list(e.want) == [0] for e in entries))
         from ..kernels import ops
         try:

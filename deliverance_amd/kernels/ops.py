@@ -12,6 +12,7 @@ from typing import Optional
 import torch
 
 from . import build
+from ..profiler import KernelProfiler
 
 F32, BF16 = 0, 1
 ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4}
@@ -97,6 +98,28 @@ def _lib():
     return _LIB
 
 
+class _NoTiming:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_TIMING = _NoTiming()
+
+
+def _timed(name: str, nbytes, flops, precision: str = "bf16"):
+    """The kernel profiler's bracket around one launch, or nothing when it is off."""
+    if not KernelProfiler.enabled:
+        return _NO_TIMING
+    return KernelProfiler.launch(name, nbytes, flops, precision)
+
+
+def _nbytes(*ts) -> int:
+    return sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+
 def _need(cond: bool, msg: str):
     if not cond:
         raise KernelError(msg)
@@ -124,8 +147,9 @@ def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
     _need(wte.is_contiguous() and wte.shape[1] == E, "embed: token table width differs from out")
     if wpe is not None:
         _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: position table width differs from out")
-    _check(_lib().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
-                                 _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, float(scale), _stream()))
+    with _timed("embed", N * E * (wte.element_size() * (2 if wpe is not None else 1) + 4), N * E, "fp32"):
+        _check(_lib().da_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _dt(wte), _ptr(wpe),
+                               _dt(wpe) if wpe is not None else 0, _ptr(out), N, E, float(scale), _stream()))
     return out
 
 
@@ -170,9 +194,10 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
         _need(R <= x.shape[0], "layernorm: more output rows than input rows")
     else:
         _need(rows.dtype == torch.int32 and rows.numel() >= R, "layernorm: rows must be int32 with R entries")
-    _check(_lib().da_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), _ptr(bias),
-                                     _dt(bias) if bias is not None else 0, eps, _ptr(out),
-                                     _dt(out), R, E, _stream()))
+    with _timed("layernorm", R * E * (4 + out.element_size()) + _nbytes(weight, bias), 8 * R * E, "fp32"):
+        _check(_lib().da_layernorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), _ptr(bias),
+                                   _dt(bias) if bias is not None else 0, eps, _ptr(out),
+                                   _dt(out), R, E, _stream()))
     return out
 
 
@@ -190,10 +215,16 @@ def linear_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], o
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
-    _check(_lib().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
-                                    _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
-                                    _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
+    with _timed("linear_ref", _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K, "fp32"):
+        _check(_lib().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
+                                  _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
+                                  _ptr(out), _dt(out), out.stride(0), M, N, K, _stream()))
     return out
+
+
+def _product_bytes(a, w, bias, out, accumulate) -> int:
+    """What a product must move at least: a, w and the bias once, the output once (twice when it adds)."""
+    return _nbytes(a, w, bias) + _nbytes(out) * (2 if accumulate else 1)
 
 
 # ------------------------------------------------------------------------------- cache write
@@ -209,8 +240,9 @@ def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.Tensor
     _need(two == 2 and Hkv == n_kv_heads and D == head_dim, "kv_write: cache slot shape differs from the heads")
     _need(cache_slot.dtype == qkv.dtype, "kv_write: cache and activations differ in dtype")
     _need(slot_map.dtype == torch.int32 and slot_map.numel() >= N, "kv_write: slot_map must be int32 [N]")
-    _check(_lib().da_kv_write(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot),
-                                    _ptr(slot_map), N, Hkv, D, page, _stream()))
+    with _timed("kv_write", 4 * N * Hkv * D * qkv.element_size(), 0, "fp32"):
+        _check(_lib().da_kv_write(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot),
+                                  _ptr(slot_map), N, Hkv, D, page, _stream()))
 
 
 # ------------------------------------------------------------------------------- attention
@@ -231,9 +263,9 @@ def attention_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.
     _need(seq_of_token.dtype == torch.int32 and positions.dtype == torch.int32, "attention: ids must be int32")
     _need(seq_of_token.numel() >= N and positions.numel() >= N, "attention: fewer ids than rows")
     _check(_lib().da_attn_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table),
-                                    block_table.shape[1], _ptr(seq_of_token), _ptr(positions), N, n_heads, Hkv,
-                                    D, page, scale, int(window or 0), _ptr(out), out.stride(0),
-                                    _stream()))
+                              block_table.shape[1], _ptr(seq_of_token), _ptr(positions), N, n_heads, Hkv,
+                              D, page, scale, int(window or 0), _ptr(out), out.stride(0),
+                              _stream()))
     return out
 
 
@@ -250,7 +282,8 @@ def sample(logits: torch.Tensor, params: torch.Tensor, out_tokens: torch.Tensor)
     _need(params.is_contiguous() and params.numel() >= R * SAMPLE_ROW_FLOATS and params.element_size() == 4,
           "sample: params must hold R records of 8 four-byte fields")
     _need(out_tokens.dtype == torch.int32 and out_tokens.numel() >= R, "sample: out must be int32 [R]")
-    _check(_lib().da_sample(_ptr(logits), logits.stride(0), R, V, _ptr(params), _ptr(out_tokens), _stream()))
+    with _timed("sample", R * V * 4, R * V, "fp32"):
+        _check(_lib().da_sample(_ptr(logits), logits.stride(0), R, V, _ptr(params), _ptr(out_tokens), _stream()))
     return out_tokens
 
 
@@ -335,9 +368,11 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
     _need(kv_cache is None or not accumulate, "linear: a cache scatter goes with a plain store")
     kvp = _kv_args(kv_cache, slot_map, q_cols, M, N, out, "linear_mfma")
-    _check(_lib().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
-                               _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
-                               _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp, _stream()))
+    name = "product_skinny" if (M <= 32 or (M <= 64 and N <= 8192)) else "product_tile"
+    with _timed(name, _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K):
+        _check(_lib().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
+                                   _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
+                                   _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp, _stream()))
     return out
 
 
@@ -381,11 +416,13 @@ def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_w
     _need(bias is None or bias.numel() == N, "linear_ln: bias length differs from N")
     _need(act in ACTIVATIONS, f"linear_ln: unknown activation {act!r}")
     kvp = _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, "linear_ln")
-    _check(_lib().da_gemm_bf16_ln(
-        _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), _ptr(norm_bias),
-        _dt(norm_bias) if norm_bias is not None else 0, eps, _ptr(w), w.stride(0), _ptr(bias),
-        _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0), n_rows, N, K,
-        *kvp, _stream()))
+    with _timed("norm_product_fused", n_rows * K * 4 + _nbytes(w, bias, norm_weight, norm_bias) + n_rows * N * out.element_size(),
+                2 * n_rows * N * K):
+        _check(_lib().da_gemm_bf16_ln(
+            _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), _ptr(norm_bias),
+            _dt(norm_bias) if norm_bias is not None else 0, eps, _ptr(w), w.stride(0), _ptr(bias),
+            _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0), n_rows, N, K,
+            *kvp, _stream()))
     return out
 
 
@@ -504,17 +541,38 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
     sequences (the first ``ctx.n_decode``) go to the decode kernel and the portions to the
     prefill kernel; 32-bit and the reference mode use the plain kernel for all rows."""
     bt = ctx.block_tables[group]
+    Hkv, page, D = cache_slot.shape[2], cache_slot.shape[3], cache_slot.shape[4]
+    el = cache_slot.element_size()
+    nd = ctx.n_decode
+    lens, starts = ctx.seq_lens_host, ctx.q_start_host        # for the profiler's cost model only
+
+    def cost(first, last):
+        """(bytes, flops) of the sequences first..last-1: every visible key and value once, q and out once;
+        two products of 2 * D flops for every (query row, visible key, head)."""
+        if not KernelProfiler.enabled or not lens:
+            return 0, 0
+        keys = pairs = rows = 0
+        for s_ in range(first, last):
+            t = starts[s_ + 1] - starts[s_]
+            n = lens[s_]
+            lo = 0 if not window else max(0, n - t - window + 1)
+            keys += n - lo
+            rows += t
+            pairs += sum(min(n - t + i + 1, window or n) for i in range(t)) if t > 1 else min(n, window or n)
+        return keys * 2 * Hkv * D * el + 2 * rows * n_heads * D * el, 4 * pairs * n_heads * D
+
     if _MODE == "tuned" and q.dtype == torch.bfloat16:
-        nd = ctx.n_decode
         if nd:
-            page, D = cache_slot.shape[3], cache_slot.shape[4]
             n_splits = decode_splits(nd, n_heads, bt.shape[1], page)
             ws = None
             if n_splits > 1:
                 ws = ctx.buf("decode_partial", 1, decode_workspace_floats(nd, n_heads, D, n_splits), torch.float32)
-            attention_decode(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, out, n_splits, ws)
+            with _timed("attention_decode", *cost(0, nd)):
+                attention_decode(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, out, n_splits, ws)
         if ctx.n_seqs > nd:
-            attention_prefill(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
-                              ctx.max_query_len, n_heads, scale, window, out)
+            with _timed("attention_prefill", *cost(nd, ctx.n_seqs)):
+                attention_prefill(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
+                                  ctx.max_query_len, n_heads, scale, window, out)
         return out
-    return attention_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, scale, window, out)
+    with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
+        return attention_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, scale, window, out)
