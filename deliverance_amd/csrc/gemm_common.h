@@ -18,7 +18,7 @@ struct Epilogue {
 };
 
 __device__ __forceinline__ void epilogue_store(const Epilogue& ep, int m, int n, float v, float bias) {
-  v = apply_act(v + bias, ep.act);
+  v = ep.out_dtype == DA_BF16 ? apply_act_bf16(v + bias, ep.act) : apply_act(v + bias, ep.act);
   const size_t o = (size_t)m * ep.ldo + n;
   if (ep.accumulate) ((float*)ep.out)[o] += v;
   else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);

@@ -175,7 +175,7 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
     for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
     epilogue_store(ep, em, n, v, e_bias[j]);
     if (kv.cache && n >= kv.q_cols && e_slot[j] >= 0)
-      kv_scatter_store(kv, e_slot[j], n, apply_act(v + e_bias[j], ep.act));
+      kv_scatter_store(kv, e_slot[j], n, apply_act_bf16(v + e_bias[j], ep.act));
   }
 }
 
@@ -335,7 +335,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
     for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
     const float e_bias = !ep.bias ? 0.f : (PBF16 ? __uint_as_float(e_bias_raw << 16) : __uint_as_float(e_bias_raw));
     epilogue_store(ep, em, en, v, e_bias);
-    if (kv.cache && en >= kv.q_cols && e_slot >= 0) kv_scatter_store(kv, e_slot, en, apply_act(v + e_bias, ep.act));
+    if (kv.cache && en >= kv.q_cols && e_slot >= 0) kv_scatter_store(kv, e_slot, en, apply_act_bf16(v + e_bias, ep.act));
   }
 }
 

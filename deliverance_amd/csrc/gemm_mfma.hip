@@ -195,7 +195,7 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
         if (m < M) {
-          const float v = apply_act(acc[i][j][r] + b, ACT);
+          const float v = OUTMODE == 0 ? apply_act_bf16(acc[i][j][r] + b, ACT) : apply_act(acc[i][j][r] + b, ACT);
           const size_t o = (size_t)m * ep.ldo + n;
           if (OUTMODE == 2) ((float*)ep.out)[o] = old[OUTMODE == 2 ? i : 0][OUTMODE == 2 ? j : 0][OUTMODE == 2 ? r : 0] + v;
           else if (OUTMODE == 1) ((float*)ep.out)[o] = v;
@@ -386,7 +386,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restri
 #pragma unroll
       for (int v2 = 1; v2 < NW; ++v2) v += red[v2][ml][c];
       const float e_bias = !ep.bias ? 0.f : (bias_bf16 ? __uint_as_float(e_braw[j] << 16) : __uint_as_float(e_braw[j]));
-      v = apply_act(v + e_bias, ep.act);
+      v = ep.out_dtype == DA_BF16 ? apply_act_bf16(v + e_bias, ep.act) : apply_act(v + e_bias, ep.act);
       const size_t o = (size_t)m * ep.ldo + n;
       if (ep.accumulate) ((float*)ep.out)[o] = e_old[j] + v;
       else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
@@ -557,7 +557,7 @@ gemm_skinny4_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restr
     v += dpp_move<0x4E, 0xF>(v, v);
     if (e_st) {
       const float e_bias = !ep.bias ? 0.f : (bias_bf16 ? __uint_as_float(e_braw << 16) : __uint_as_float(e_braw));
-      v = apply_act(v + e_bias, ep.act);
+      v = ep.out_dtype == DA_BF16 ? apply_act_bf16(v + e_bias, ep.act) : apply_act(v + e_bias, ep.act);
       const size_t o = (size_t)e_m * ep.ldo + e_n;
       if (ep.accumulate) ((float*)ep.out)[o] = e_old + v;
       else if (ep.out_dtype == DA_BF16) ((bf16_t*)ep.out)[o] = f32_to_bf16(v);

@@ -102,6 +102,7 @@ int dpp_source(int lane, int ctrl);    // the lane a DPP control reads from, or 
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 
 static inline int simt_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool) {
   const int lane = simt::lane_id();

@@ -29,7 +29,7 @@ def test_random_then_inspect(tmp_path):
 def test_help_names_the_reference_options():
     p = run("generate", "--help")
     for opt in ("--model", "--working-dtype", "--max-tokens", "--temperature", "--seed", "--warmup-cases", "--max-cases",
-                "--kv-context-rows-per-page", "--model-config", "--profile-stages", "--suite-file", "--output", "--jsonl-output"):
+                "--kv-context-rows-per-page", "--model-config", "--profile-stages", "--kernels", "--suite-file", "--output", "--jsonl-output"):
         assert opt in p.stdout
     p = run("generate", "--model", "/nonexistent")
     assert p.returncode != 0

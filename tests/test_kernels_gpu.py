@@ -127,12 +127,13 @@ def test_gemm_plain_32bit(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 3, 5, 8, 12, 16, 17, 40, 64, 65, 128, 200, 513, 1100, 2048])
-@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24), (300, 2056), (1030, 1160)])
+@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24), (300, 2056), (1030, 1160), (4200, 200),
+                                 (4096, 8)])
 def test_gemm_matrix_cores(ops, M, N, K):
     """Every kernel form behind ``linear_mfma`` (up to 4 rows and 2,048 columns: 4x4x4 products, 4 to 16
     wavefronts; up to 64 rows: 16x16x32 products fed through LDS, 1 to 4 row tiles, 8 or 12 wavefronts;
     else block tiles of 64x64, 128x64 and 128x128, chosen by the number of tiles: 1,100 and 2,048 rows
-    reach the larger ones), each with a last step that K cuts."""
+    reach the larger ones), each with a last step that K cuts or a K below one slab."""
     helpers.skip_in_simulation_if(M * N * K > 1.2e8)
     g = torch.Generator().manual_seed(M * 7 + N)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),

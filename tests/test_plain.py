@@ -112,6 +112,13 @@ def test_block_structure(model_a):
 
 
 def test_fused_projection_is_three_projections_in_q_k_v_order(model_b):
+    """The plain attention block is its parts put together: the fused projection's columns taken as
+    thirds q | k | v (core/src/main/java/io/teknek/deliverance/model/gpt2/Gpt2Model.java:81-82 slices
+    c_attn in that order), attention, output projection.  Parity unpinned: the reference holds no vector
+    for GPT-2's attention block, so the ORDER of the thirds rests on reading those two lines; what this
+    test can catch is a plain block whose parts are not wired as its own functions say (a swapped k and
+    v shows: the result below changes by far more than rounding), and the engine's order is held to the
+    plain model's by every replay test."""
     cfg, W = model_b.plain_cfg, model_b.W
     E, H = cfg["n_embd"], cfg["n_head"]
     rng = np.random.default_rng(5)
@@ -122,6 +129,8 @@ def test_fused_projection_is_three_projections_in_q_k_v_order(model_b):
     o = P.causal_attention(q, k, v, H, scale)
     want = o @ W["h.1.attn.c_proj.weight"] + W["h.1.attn.c_proj.bias"]
     assert np.abs(P.attention_block(a, W, 1, H, scale) - want).max() < 1e-12
+    swapped = P.causal_attention(q, v, k, H, scale) @ W["h.1.attn.c_proj.weight"] + W["h.1.attn.c_proj.bias"]
+    assert np.abs(swapped - want).max() > 1e-3
 
 
 def test_whole_model_properties(model_a, model_b):
