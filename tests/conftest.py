@@ -18,6 +18,10 @@ SIMT = os.environ.get("DELIVERANCE_SIMT") == "1"
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
     config.addinivalue_line("markers", "needs_device: a GPU test that cannot run on the simulated kernels")
+    # the selection of GPU test cases that tests/test_simt.py runs on the simulated kernels by default: simt_quick, or,
+    # where two parameter lists cross, a case marked on both (simt_a and simt_b)
+    for m in ("simt_quick", "simt_a", "simt_b"):
+        config.addinivalue_line("markers", f"{m}: part of the default selection for the simulated kernels")
 
 
 def pytest_collection_modifyitems(config, items):

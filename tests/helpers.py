@@ -36,6 +36,12 @@ def trace_session(folder, dtype, max_tokens, page_size=16, poison_freed=False, *
     return TraceSession(str(folder), dtype, max_tokens, page_size, poison_freed=poison_freed, **options)
 
 
+def quick(*values, mark="simt_quick"):
+    """A parameter of the default selection for the simulated kernels (tests/test_simt.py)."""
+    import pytest
+    return pytest.param(*values, marks=getattr(pytest.mark, mark))
+
+
 def skip_in_simulation_if(cond, why="too much arithmetic for the simulated kernels"):
     if SIMT and cond:
         import pytest

@@ -26,6 +26,7 @@ def bf(x):
 
 
 # ----------------------------------------------------------------------------- embedding, norm
+@pytest.mark.simt_quick
 @pytest.mark.parametrize("table_dtype", [torch.float32, torch.bfloat16])
 def test_embed(ops, table_dtype):
     g = torch.Generator().manual_seed(0)
@@ -42,6 +43,7 @@ def test_embed(ops, table_dtype):
     assert torch.equal(out, wte.float()[tok.long()])
 
 
+@pytest.mark.simt_quick
 def test_embed_scale_and_row_copies(ops):
     g = torch.Generator().manual_seed(2)
     V, Pn, E, N = 300, 50, 72, 21
@@ -68,6 +70,7 @@ def test_embed_scale_and_row_copies(ops):
         ops.copy_rows(out, bf(out), accumulate=True)
 
 
+@pytest.mark.simt_quick
 @pytest.mark.parametrize("E,eps", [(7, 1e-5), (200, 1e-6), (1600, 1e-5), (64, 1e-1)])
 def test_layernorm(ops, E, eps):
     g = torch.Generator().manual_seed(1)
@@ -117,6 +120,7 @@ def _gemm_case(ops, fn, M, N, K, dtype, act, accumulate, bias, out_dtype, g):
     return out.double(), ref
 
 
+@pytest.mark.simt_quick
 @pytest.mark.parametrize("M,N,K", [(1, 50, 24), (5, 1000, 96), (70, 200, 96), (130, 77, 200), (64, 64, 64)])
 def test_gemm_plain_32bit(ops, M, N, K):
     g = torch.Generator().manual_seed(M * 1000 + N)
@@ -126,9 +130,11 @@ def test_gemm_plain_32bit(ops, M, N, K):
         assert (out - ref).abs().max() < 2e-5 * max(1.0, ref.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [1, 3, 5, 8, 12, 16, 17, 40, 64, 65, 128, 200, 513, 1100, 2048])
-@pytest.mark.parametrize("N,K", [(96, 200), (1000, 96), (2304, 768), (50, 24), (300, 2056), (1030, 1160), (4200, 200),
-                                 (4096, 8)])
+@pytest.mark.parametrize("M", [1, helpers.quick(3, mark="simt_a"), 5, 8, 12, 16, helpers.quick(17, mark="simt_a"), 40, 64,
+                               helpers.quick(65, mark="simt_a"), 128, helpers.quick(200, mark="simt_a"), 513, 1100, 2048])
+@pytest.mark.parametrize("N,K", [helpers.quick(96, 200, mark="simt_b"), helpers.quick(1000, 96, mark="simt_b"), (2304, 768),
+                                 helpers.quick(50, 24, mark="simt_b"), helpers.quick(300, 2056, mark="simt_b"), (1030, 1160),
+                                 (4200, 200), helpers.quick(4096, 8, mark="simt_b")])
 def test_gemm_matrix_cores(ops, M, N, K):
     """Every kernel form behind ``linear_mfma`` (up to 4 rows and 2,048 columns: 4x4x4 products, 4 to 16
     wavefronts; up to 64 rows: 16x16x32 products fed through LDS, 1 to 4 row tiles, 8 or 12 wavefronts;
@@ -144,6 +150,7 @@ def test_gemm_matrix_cores(ops, M, N, K):
         assert (out - ref).abs().max() < tol, (act, acc, bias, od)
 
 
+@pytest.mark.simt_quick
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """A row's result is the same, bit for bit, whatever other rows share the call, as long as the call
     takes the same kernel form (block tiles; 16x16x32 products up to 64 rows; 4x4x4 products up to 4
@@ -172,6 +179,7 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
         assert (f.double() - exact).abs().max() < 2e-6 * scale
 
 
+@pytest.mark.simt_quick
 def test_gemm_refuses_what_it_cannot_take(ops):
     a = torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16)
     w = torch.zeros(8, 12, device=DEV, dtype=torch.bfloat16)
@@ -238,7 +246,7 @@ ATT_TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [helpers.quick(4, 4, 16, 16, None), (6, 2, 48, 16, None), helpers.quick(2, 1, 80, 32, 37),
                                                   (3, 3, 128, 64, None), (5, 5, 64, 16, 100)])
 def test_attention_plain_kernel(ops, dtype, Hq, Hkv, D, page, window):
     case = PagedCase(lens=[70, 5, 131, 64], new=[70, 1, 9, 2], Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=dtype, seed=D)
@@ -248,9 +256,9 @@ def test_attention_plain_kernel(ops, dtype, Hq, Hkv, D, page, window):
     assert np.abs(out.double().cpu().numpy() - case.plain(scale, window)).max() < ATT_TOL[dtype]
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [helpers.quick(4, 4, 16, 16, None), (6, 2, 48, 16, None), helpers.quick(2, 1, 80, 32, 37),
                                                   (3, 3, 128, 64, None), (12, 12, 64, 16, None), (5, 5, 64, 16, 100),
-                                                  (2, 2, 256, 16, None), (25, 25, 64, 32, 70)])
+                                                  helpers.quick(2, 2, 256, 16, None), (25, 25, 64, 32, 70)])
 def test_attention_decode_kernel(ops, Hq, Hkv, D, page, window):
     lens = [1, 2, 63, 64, 65, 300, 129, 17, 1000]
     case = PagedCase(lens=lens, new=[1] * len(lens), Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + 1)
@@ -262,9 +270,9 @@ def test_attention_decode_kernel(ops, Hq, Hkv, D, page, window):
     assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
 
 
-@pytest.mark.parametrize("n_splits", [2, 3, 7, 16])
-@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(2, 2, 64, 16, None), (4, 2, 48, 32, None), (1, 1, 128, 64, 700),
-                                                  (3, 3, 16, 16, 90)])
+@pytest.mark.parametrize("n_splits", [2, helpers.quick(3, mark="simt_a"), 7, 16])
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [helpers.quick(2, 2, 64, 16, None, mark="simt_b"), (4, 2, 48, 32, None),
+                                                  helpers.quick(1, 1, 128, 64, 700, mark="simt_b"), (3, 3, 16, 16, 90)])
 def test_attention_decode_with_keys_split_over_workgroups(ops, Hq, Hkv, D, page, window, n_splits):
     """Every (sequence, head) pair's keys in ``n_splits`` shares with a merge in a fixed order: shares
     that hold nothing (short sequences, a window that has passed them), one key, a share's first and
@@ -288,6 +296,7 @@ def test_attention_decode_with_keys_split_over_workgroups(ops, Hq, Hkv, D, page,
         ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, out, n_splits, ws[:10])
 
 
+@pytest.mark.simt_quick
 def test_when_decode_attention_splits_its_keys(ops):
     assert ops.decode_splits(1, 12, 64, 16) == 1                   # 1,024 keys: one share
     assert ops.decode_splits(1, 12, 256, 16) == 4                  # 4,096 keys, 12 pairs: shares of 1,024
@@ -296,9 +305,9 @@ def test_when_decode_attention_splits_its_keys(ops):
     assert ops.decode_splits(1, 1, 4096, 16) == 32                 # never more than 32
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), (6, 2, 48, 16, None), (2, 1, 80, 32, 37),
+@pytest.mark.parametrize("Hq,Hkv,D,page,window", [(4, 4, 16, 16, None), helpers.quick(6, 2, 48, 16, None), helpers.quick(2, 1, 80, 32, 37),
                                                   (3, 3, 128, 64, None), (12, 12, 64, 16, None), (5, 5, 64, 16, 100),
-                                                  (2, 2, 256, 16, None), (2, 2, 240, 16, None), (3, 1, 64, 32, 200)])
+                                                  (2, 2, 256, 16, None), (2, 2, 240, 16, None), helpers.quick(3, 1, 64, 32, 200)])
 def test_attention_prefill_kernel(ops, Hq, Hkv, D, page, window):
     lens = [70, 200, 131, 64, 2, 300, 513]
     new = [70, 9, 131, 2, 2, 129, 260]            # whole prompts, short portions after a long past, tiles' edges
@@ -312,6 +321,7 @@ def test_attention_prefill_kernel(ops, Hq, Hkv, D, page, window):
     assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
 
 
+@pytest.mark.simt_quick
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_a_row_that_sees_no_key_gives_zeros(ops, dtype):
     """The padding rows of a fixed-shape decode step: length 0, a block table of -1.  Zeros, never NaN
@@ -335,6 +345,7 @@ def test_a_row_that_sees_no_key_gives_zeros(ops, dtype):
         assert np.abs(out2[:2].double().cpu().numpy() - want).max() < ATT_TOL[dtype]
 
 
+@pytest.mark.simt_quick
 def test_attention_reference_vector_shape(ops):
     """The shape of the reference's own paged-attention test: 4 query heads on 2 key heads, head 8
     there (16 here: head sizes come in steps of 16), pages of 3 rows there (16 here), 5 visible rows,
@@ -366,6 +377,7 @@ def test_attention_reference_vector_shape(ops):
             assert np.abs(out2.double().cpu().numpy() - want).max() < tol
 
 
+@pytest.mark.simt_quick
 @pytest.mark.parametrize("page", [16, 32, 64])
 @pytest.mark.parametrize("N", [40, 600])
 def test_cache_write_puts_every_key_and_value_in_its_row(ops, N, page):
@@ -464,6 +476,7 @@ def test_sampling_kernel_against_the_plain_sampler(ops):
         assert got[r] == want, (r, p)
 
 
+@pytest.mark.simt_quick
 def test_sampling_vectors_of_the_reference(ops):
     """core/src/test/java/io/teknek/deliverance/model/TopKSamplerTest.java:23-54, with the draws given."""
     import struct
@@ -480,6 +493,7 @@ def test_sampling_vectors_of_the_reference(ops):
     assert out.cpu().tolist() == [1, 0, 1, 0, 4, 0, 2]
 
 
+@pytest.mark.simt_quick
 def test_xtc_and_logprobs(ops):
     import struct
     V = 1000
@@ -506,9 +520,9 @@ def test_xtc_and_logprobs(ops):
 
 
 # ----------------------------------------------------------------------------- fused norm + product
-@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 2304, 768), (17, 1000, 96), (32, 200, 1600), (5, 50257, 768),
-                                   (16, 520, 1024), (12, 72, 1000), (9, 40, 520), (3, 1000, 1600), (16, 300, 2048),
-                                   (5, 64, 1304), (2, 48, 8), (11, 200, 1992)])
+@pytest.mark.parametrize("M,N,K", [helpers.quick(1, 96, 64), (8, 2304, 768), helpers.quick(17, 1000, 96), (32, 200, 1600), (5, 50257, 768),
+                                   (16, 520, 1024), helpers.quick(12, 72, 1000), helpers.quick(9, 40, 520), (3, 1000, 1600), (16, 300, 2048),
+                                   helpers.quick(5, 64, 1304), helpers.quick(2, 48, 8), (11, 200, 1992)])
 @pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_product(ops, M, N, K, pdtype):
     helpers.skip_in_simulation_if(M * N * K > 1.2e8)
@@ -531,7 +545,7 @@ def test_fused_norm_product(ops, M, N, K, pdtype):
         assert (out.double() - ref).abs().max() < tol
 
 
-@pytest.mark.parametrize("M", [5, 40, 300])
+@pytest.mark.parametrize("M", [helpers.quick(5), helpers.quick(40), 300])
 def test_product_writes_keys_and_values(ops, M):
     """The skinny (M <= 64) and tile kernels scatter the k | v columns in their epilogue."""
     g = torch.Generator().manual_seed(M)
@@ -555,6 +569,7 @@ def test_product_writes_keys_and_values(ops, M):
     assert torch.equal(c1, c2) and c1.abs().sum() > 0
 
 
+@pytest.mark.simt_quick
 def test_fused_norm_product_writes_keys_and_values(ops):
     g = torch.Generator().manual_seed(11)
     Hq, Hkv, D, page, M, K = 6, 2, 48, 16, 9, 96
