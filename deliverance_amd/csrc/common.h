@@ -48,10 +48,9 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
 // Round to nearest even; NaN stays a quiet NaN (the reference's C side rounds the same
 // way: native/src/main/c/simd/vector_simd.c:23-41, except that it flushes subnormals).
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16, quiet = (u >> 16) | 0x0040u;
+  return (bf16_t)((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded);      // a select, not a branch
 }
 
 // Two floats to two bfloat16 in one word (first in the low half), round to nearest even, by the

@@ -34,12 +34,17 @@ struct KvScatter {
   int Hkv, D, page;
 };
 
-__device__ __forceinline__ void kv_scatter_store(const KvScatter& kv, int slot, int n, float v) {
+// column n (>= q_cols) of a row whose place in the cache is row `row` of page `pg`
+__device__ __forceinline__ void kv_scatter_bits(const KvScatter& kv, int pg, int row, int n, bf16_t bits) {
   const int c2 = n - kv.q_cols, is_v = c2 >= kv.kv_cols, cc = is_v ? c2 - kv.kv_cols : c2;
-  const int h = cc / kv.D, d = cc % kv.D, pg = slot / kv.page, row = slot % kv.page;
+  const int h = cc / kv.D, d = cc % kv.D;
   bf16_t* cache = (bf16_t*)kv.cache;
-  if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = f32_to_bf16(v);
-  else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = f32_to_bf16(v);
+  if (is_v) cache[cache_v_base(pg, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + row] = bits;
+  else cache[cache_k_row(pg, h, row, kv.Hkv, kv.page, kv.D) + d] = bits;
+}
+
+__device__ __forceinline__ void kv_scatter_store(const KvScatter& kv, int slot, int n, float v) {
+  kv_scatter_bits(kv, slot / kv.page, slot % kv.page, n, f32_to_bf16(v));
 }
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }

@@ -34,11 +34,130 @@
 // ---------------------------------------------------------------------------------------------
 // OUTMODE: 0 bf16 store, 1 f32 store, 2 f32 +=.  ACT and OUTMODE are compile-time so that the
 // epilogue is straight-line code.
+// ---------------------------------------------------------------------------------------------
+// The epilogue of a block tile.  A lane holds one column and 16 scattered rows of each 32 x 32 piece,
+// two or four bytes wide: stored from there, a wavefront's store covers 64 bytes a row.  Instead the
+// workgroup parks the tile in LDS (bias and activation applied, rounded to the output's type) and
+// stores it row by row in 16-byte pieces, a whole row of the tile side by side; what += adds to is
+// loaded the same way.  All loads come first and are used in straight-line code, only stores stand
+// under conditions: a load under a condition would make each store wait for the one before it.
+// OUTMODE: 0 bf16 store, 1 f32 store, 2 f32 +=.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int OUTMODE>
+constexpr int tile_out_bytes() {
+  return BM * (BN + (OUTMODE == 0 ? 8 : 4)) * (OUTMODE == 0 ? 2 : 4);
+}
+
+template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
+__device__ __forceinline__ void
+tile_epilogue(floatx16 (&acc)[BM / WM / 32][BN / WN / 32], const float (&bias)[BN / WN / 32], char* smem, const void* safe,
+              const Epilogue& ep, const KvScatter& kv, int M, int N, int m0, int n0) {
+  constexpr int THREADS = WM * WN * 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int ES = OUTMODE == 0 ? 2 : 4, CH = 16 / ES;      // bytes an element; elements a 16-byte piece
+  constexpr int LDT = BN + CH;                                 // a parked row, padded by one piece
+  constexpr int CPR = BN / CH, NCHK = BM * CPR / THREADS;      // pieces a row; pieces a thread
+  static_assert(BM * CPR % THREADS == 0, "the tile's pieces do not split over the threads");
+  const int t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int wm = (wave % WM) * (BM / WM), wn = (wave / WM) * (BN / WN);
+  const int fr = lane % 32;
+
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int nl = wn + j * 32 + fr;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ml = wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (OUTMODE == 0) ((bf16_t*)smem)[ml * LDT + nl] = f32_to_bf16(apply_act_bf16(acc[i][j][r] + bias[j], ACT));
+        else ((float*)smem)[ml * LDT + nl] = apply_act(acc[i][j][r] + bias[j], ACT);
+      }
+  }
+  lds_barrier();
+
+  uint4 val[NCHK];
+  int mm[NCHK], nn[NCHK];
+#pragma unroll
+  for (int k = 0; k < NCHK; ++k) {
+    const int q = t + THREADS * k, row = q / CPR, c = q % CPR;
+    mm[k] = m0 + row;
+    nn[k] = n0 + c * CH;
+    val[k] = *(const uint4*)(smem + (size_t)(row * LDT + c * CH) * ES);
+  }
+  const bool wide = (uintptr_t)ep.out % 16 == 0 && ep.ldo % CH == 0;
+  if (wide) {
+    if (OUTMODE == 2) {
+      uint4 old[NCHK];
+#pragma unroll
+      for (int k = 0; k < NCHK; ++k) {
+        const bool whole = mm[k] < M && nn[k] + CH <= N;
+        old[k] = *(const uint4*)(whole ? (const void*)((const float*)ep.out + (size_t)mm[k] * ep.ldo + nn[k]) : safe);
+      }
+#pragma unroll
+      for (int k = 0; k < NCHK; ++k) {
+        const bool whole = mm[k] < M && nn[k] + CH <= N;     // (a select: what came from the safe place is dropped)
+        val[k].x = whole ? __float_as_uint(__uint_as_float(old[k].x) + __uint_as_float(val[k].x)) : val[k].x;
+        val[k].y = whole ? __float_as_uint(__uint_as_float(old[k].y) + __uint_as_float(val[k].y)) : val[k].y;
+        val[k].z = whole ? __float_as_uint(__uint_as_float(old[k].z) + __uint_as_float(val[k].z)) : val[k].z;
+        val[k].w = whole ? __float_as_uint(__uint_as_float(old[k].w) + __uint_as_float(val[k].w)) : val[k].w;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NCHK; ++k)
+      if (mm[k] < M && nn[k] + CH <= N) *(uint4*)((char*)ep.out + ((size_t)mm[k] * ep.ldo + nn[k]) * ES) = val[k];
+  }
+  // pieces that N cuts, and everything where the output's rows are not 16-byte aligned: by elements
+  // (for +=, a piece that N cuts still holds the bare products here: only whole pieces were added to above)
+#pragma unroll
+  for (int k = 0; k < NCHK; ++k) {
+    if (mm[k] >= M || nn[k] >= N || (wide && nn[k] + CH <= N)) continue;
+    const uint32_t words[4] = {val[k].x, val[k].y, val[k].z, val[k].w};
+#pragma unroll
+    for (int e = 0; e < CH; ++e) {
+      if (nn[k] + e >= N) continue;
+      const size_t o = (size_t)mm[k] * ep.ldo + nn[k] + e;
+      if (OUTMODE == 0) ((bf16_t*)ep.out)[o] = (bf16_t)(words[e / 2] >> (16 * (e % 2)));
+      else if (OUTMODE == 1) ((float*)ep.out)[o] = __uint_as_float(words[e % 4]);
+      else ((float*)ep.out)[o] += __uint_as_float(words[e % 4]);
+    }
+  }
+
+  // a fused q|k|v projection: the k and v columns also go to the rows' places in the paged cache
+  if (OUTMODE == 0 && kv.cache) {
+    int pg[NCHK], prow[NCHK];
+#pragma unroll
+    for (int k = 0; k < NCHK; ++k) {
+      const int slot = kv.slot_map[mm[k] < M ? mm[k] : M - 1];
+      pg[k] = slot < 0 ? -1 : slot / kv.page;
+      prow[k] = slot < 0 ? 0 : slot % kv.page;
+    }
+    const bool kwide = (uintptr_t)kv.cache % 16 == 0 && kv.D % 8 == 0 && kv.q_cols % 8 == 0;
+#pragma unroll
+    for (int k = 0; k < NCHK; ++k) {
+      if (mm[k] >= M || nn[k] >= N || nn[k] + 8 <= kv.q_cols || pg[k] < 0) continue;
+      const int c2 = nn[k] - kv.q_cols;
+      if (kwide && c2 < kv.kv_cols) {           // eight dimensions of one key: one piece of its row
+        const int h = c2 / kv.D, d = c2 % kv.D;
+        *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg[k], h, prow[k], kv.Hkv, kv.page, kv.D) + d) = val[k];
+        continue;
+      }
+      const uint32_t words[4] = {val[k].x, val[k].y, val[k].z, val[k].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (nn[k] + e < N && nn[k] + e >= kv.q_cols)
+          kv_scatter_bits(kv, pg[k], prow[k], nn[k] + e, (bf16_t)(words[e / 2] >> (16 * (e % 2))));
+    }
+  }
+}
+
 template <int BM, int BN, int WM, int WN, int PF_SLABS, int ACT, int OUTMODE, bool KTAIL>
 __device__ __forceinline__ void
 gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                const Epilogue& ep, const KvScatter& kv, int M, int N, int K, int tiles_m, int tiles_n,
-               bf16_t (*As)[BM * LDS_LD], bf16_t (*Ws)[BN * LDS_LD]) {
+               char* smem) {
+  bf16_t (*As)[BM * LDS_LD] = (bf16_t (*)[BM * LDS_LD])smem;
+  bf16_t (*Ws)[BN * LDS_LD] = (bf16_t (*)[BN * LDS_LD])(smem + 2 * BM * LDS_LD * sizeof(bf16_t));
   constexpr int THREADS = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;       // MFMA tiles per wavefront
   constexpr int CA = BM * 8 / THREADS, CW = BN * 8 / THREADS; // 16-byte chunks per thread and slab
@@ -118,22 +237,18 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
   }
   const int fr = lane % 32, fk = (lane / 32) * 8;
   const int nslab = (K + BKT - 1) / BKT;
-  // what the output held before (+=) is asked for now, from clamped places, and has long arrived
-  // when the products are done
-  float old[OUTMODE == 2 ? TM : 1][OUTMODE == 2 ? TN : 1][OUTMODE == 2 ? 16 : 1];
-  if (OUTMODE == 2) {
+  // The bias is asked for now, as raw bits from a place that always exists, and has long arrived when
+  // the products are done: a load inside the epilogue's conditions would make every store after it
+  // wait for the one before.
+  const bool bias_bf16 = ep.bias_dtype == DA_BF16;
+  uint32_t braw[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn + j * 32 + fr, nc = n < N ? n : N - 1;
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4), mc = m < M ? m : M - 1;
-          old[OUTMODE == 2 ? i : 0][OUTMODE == 2 ? j : 0][OUTMODE == 2 ? r : 0] =
-              ((const float*)ep.out)[(size_t)mc * ep.ldo + nc];
-        }
-    }
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn + j * 32 + fr;
+    const bool has = ep.bias && n < N;
+    const void* src = has ? ep.bias : (const void*)w;
+    const int idx = has ? n : 0;
+    braw[j] = bias_bf16 ? (uint32_t)((const bf16_t*)src)[idx] : ((const uint32_t*)src)[idx];
   }
 #pragma unroll
   for (int j = 0; j < PF_SLABS; ++j)
@@ -184,39 +299,22 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
 #undef TILE_FETCH
 #undef TILE_STASH
 
+  float bias[TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn + j * 32 + fr;
-    if (n >= N) continue;
-    const float b = ep.bias ? load_param(ep.bias, ep.bias_dtype, n) : 0.f;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-        if (m < M) {
-          const float v = OUTMODE == 0 ? apply_act_bf16(acc[i][j][r] + b, ACT) : apply_act(acc[i][j][r] + b, ACT);
-          const size_t o = (size_t)m * ep.ldo + n;
-          if (OUTMODE == 2) ((float*)ep.out)[o] = old[OUTMODE == 2 ? i : 0][OUTMODE == 2 ? j : 0][OUTMODE == 2 ? r : 0] + v;
-          else if (OUTMODE == 1) ((float*)ep.out)[o] = v;
-          else ((bf16_t*)ep.out)[o] = f32_to_bf16(v);
-          if (OUTMODE == 0 && kv.cache && n >= kv.q_cols) {
-            const int slot = kv.slot_map[m];
-            if (slot >= 0) kv_scatter_store(kv, slot, n, v);
-          }
-        }
-      }
-  }
+  for (int j = 0; j < TN; ++j) bias[j] = !ep.bias ? 0.f : (bias_bf16 ? __uint_as_float(braw[j] << 16) : __uint_as_float(braw[j]));
+  tile_epilogue<BM, BN, WM, WN, ACT, OUTMODE>(acc, bias, smem, (const void*)w, ep, kv, M, N, m0, n0);
 }
 
 template <int BM, int BN, int WM, int WN, int PF, int ACT, int OUTMODE>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                  Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_LD];      // shared by the two bodies
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_LD];
-  if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, As, Ws);
-  else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, As, Ws);
+  // two buffers of a slab of a and of w; the epilogue parks the tile's results in the same memory
+  constexpr int SLAB_BYTES = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16_t);
+  constexpr int OUT_BYTES = tile_out_bytes<BM, BN, OUTMODE>();
+  __shared__ __attribute__((aligned(16))) char smem[SLAB_BYTES > OUT_BYTES ? SLAB_BYTES : OUT_BYTES];      // shared by the two bodies
+  if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);
+  else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);
 }
 
 template <int BM, int BN, int WM, int WN, int PF, int ACT>
