@@ -187,17 +187,24 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 // steps v, v + 8, ...) are asked for before anything else is computed and parked in the wavefront's
 // own piece of LDS; the fragments of both operands are read from LDS.  Steps past K read step 0 and
 // meet zeros.  The sum over k runs in the order of the steps, whatever M is.
+// TWO_ROWS false: M <= 8, a wavefront has one row and LDS holds 8 (the fragment's rows 8..15 read
+// rows 0..7 again and are never stored): half the LDS, so that with a wide K two workgroups still
+// share a compute unit and N / 16 workgroups run side by side.
 // ---------------------------------------------------------------------------------------------
 #define FL_LD (64 + 8)       // padded row of a parked step of w, elements
-template <int RV, bool PBF16>
+template <int RV, bool PBF16, bool TWO_ROWS>
 __global__ void __launch_bounds__(512)
 gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
                    int M, int N, int K) {
   constexpr int NW = 8, KMAX = RV * 256, ALD = KMAX + 8;      // ALD: padded row of a in LDS, elements
   constexpr int SW = (RV * 4 + NW - 1) / NW;                   // steps a wavefront
-  __shared__ __attribute__((aligned(16))) bf16_t a_lds[16][ALD];
-  __shared__ __attribute__((aligned(16))) bf16_t stage[NW][16 * FL_LD];
-  __shared__ float red[NW][16][FZ_COLS + 1];
+  constexpr int RPW = TWO_ROWS ? 2 : 1, AR = RPW * NW;         // rows a wavefront normalises; rows in LDS
+  __shared__ __attribute__((aligned(16))) bf16_t a_lds[AR][ALD];
+  // the wavefronts' sums take the place of the parked steps once all products are done
+  constexpr int STAGE_BYTES = NW * 16 * FL_LD * 2, RED_BYTES = NW * 16 * (FZ_COLS + 1) * 4;
+  __shared__ __attribute__((aligned(16))) char stage_red[STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES];
+  bf16_t (*stage)[16 * FL_LD] = (bf16_t (*)[16 * FL_LD])stage_red;
+  float (*red)[16][FZ_COLS + 1] = (float (*)[16][FZ_COLS + 1])stage_red;
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int n0 = blockIdx.x * FZ_COLS;
   const int fr = lane % 16, fk = (lane / 16) * 8;    // a fragment: row fr of 16, k-group lane / 16
@@ -207,10 +214,10 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
   // (rows from M on are neither read nor normalised: what they give is never stored; the row number
   // is made a scalar so that the branch around their loads is one for the whole wavefront)
   const int row0 = __builtin_amdgcn_readfirstlane(wave);
-  float4 sv[2][RV];
+  float4 sv[RPW][RV];
   uint4 gq[RV], bq[RV];                              // gain and bias at this lane's places (bfloat16: .x .y only)
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < RPW; ++j) {
     const int m = row0 + j * NW;
     if (m < M) {
       const float* xr = ln.x + (size_t)(ln.rows ? ln.rows[m] : m) * K;
@@ -257,7 +264,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
 
   // ---- statistics and the normalised rows
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < RPW; ++j) {
     const int m = row0 + j * NW;
     if (m >= M) continue;
     float sum = 0.f;
@@ -318,7 +325,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
 #pragma unroll
       for (int c = 0; c < 64; c += 32) {
         const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[fr * FL_LD + c + fk]);
-        const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&a_lds[fr][k0 + c + fk]);
+        const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&a_lds[fr % AR][k0 + c + fk]);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc, 0, 0, 0);
       }
     }
@@ -326,6 +333,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
+  lds_barrier();                                     // every wavefront is done with its parked steps
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][4 * (lane / 16) + r][fr] = acc[r];
   lds_barrier();
@@ -371,19 +379,28 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
   // the kernel with whole-line loads takes one row tile, K up to 2048, and parameters of one dtype
   const int pdt = g_dtype;
   const bool same = (!b || b_dtype == pdt) && (!bias || bias_dtype == pdt) && (pdt == DA_BF16 || pdt == DA_F32);
+#define LAUNCH_LDS_P(RV, PB)                                                                                      \
+  do {                                                                                                            \
+    if (M <= 8)                                                                                                   \
+      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, PB, false>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+    else                                                                                                          \
+      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, PB, true>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+  } while (0)
 #define LAUNCH_LDS(RV)                                                                                            \
   do {                                                                                                            \
     if (pdt == DA_BF16)                                                                                           \
-      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, true>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+      LAUNCH_LDS_P(RV, true);                                                                                     \
     else                                                                                                          \
-      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, false>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+      LAUNCH_LDS_P(RV, false);                                                                                    \
   } while (0)
   if (mt == 1 && same && K <= 2048) {
     if (K <= 256) LAUNCH_LDS(1);
     else if (K <= 512) LAUNCH_LDS(2);
     else if (K <= 768) LAUNCH_LDS(3);
     else if (K <= 1024) LAUNCH_LDS(4);
+    else if (K <= 1280) LAUNCH_LDS(5);
     else if (K <= 1536) LAUNCH_LDS(6);
+    else if (K <= 1792) LAUNCH_LDS(7);
     else LAUNCH_LDS(8);
   } else
     // 8 wavefronts, two chunks in flight each: 125 registers, so two workgroups share a compute unit

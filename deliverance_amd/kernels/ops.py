@@ -377,11 +377,11 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 
 # Measured on MI355X inside the model: the fused kernel wins up to 16 rows (one row tile) and a
-# width of 1024, by 10 to 15 % of a decode step; beyond, the separate norm and product are faster
-# (every 16 output columns recompute the rows' statistics, and a wavefront's loads come in more
-# rounds).
-FUSED_LN_MAX_ROWS = 16
-FUSED_LN_MAX_K = 1024
+# width of 1024, by 10 to 15 % of a decode step; up to 8 rows (which take half the LDS, so that the
+# workgroups still run side by side) up to a width of 1280, and a single row up to 2048; beyond, the
+# separate norm and product are faster (every 16 output columns read and normalise all rows again:
+# at a width of 1600 and 8 rows 8.0 us against 3.1 + 3.9).
+FUSED_LN_LIMITS = ((16, 1024), (8, 1280), (1, 2048))       # (rows, width): fused up to these
 FUSED_LN_MAX_N = 16384      # ... and never for a vocabulary
 FUSED_LN_KERNEL_MAX_ROWS = 32
 
@@ -389,8 +389,9 @@ FUSED_LN_KERNEL_MAX_ROWS = 32
 def can_fuse_ln(n_rows: int, x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether ``linear_ln`` takes this step: few rows, bfloat16 weights, a width the kernel holds."""
     K = w.shape[1]
-    return (_MODE == "tuned" and w.dtype == torch.bfloat16 and 0 < n_rows <= FUSED_LN_MAX_ROWS
-            and K % 8 == 0 and K <= FUSED_LN_MAX_K and w.shape[0] <= FUSED_LN_MAX_N
+    fits = any(n_rows <= r and K <= k for r, k in FUSED_LN_LIMITS)
+    return (_MODE == "tuned" and w.dtype == torch.bfloat16 and 0 < n_rows and fits
+            and K % 8 == 0 and w.shape[0] <= FUSED_LN_MAX_N
             and w.stride(0) % 8 == 0 and x.dtype == torch.float32)
 
 

@@ -522,7 +522,8 @@ def test_xtc_and_logprobs(ops):
 # ----------------------------------------------------------------------------- fused norm + product
 @pytest.mark.parametrize("M,N,K", [helpers.quick(1, 96, 64), (8, 2304, 768), helpers.quick(17, 1000, 96), (32, 200, 1600), (5, 50257, 768),
                                    (16, 520, 1024), helpers.quick(12, 72, 1000), helpers.quick(9, 40, 520), (3, 1000, 1600), (16, 300, 2048),
-                                   helpers.quick(5, 64, 1304), helpers.quick(2, 48, 8), (11, 200, 1992)])
+                                   helpers.quick(5, 64, 1304), helpers.quick(2, 48, 8), (11, 200, 1992), (8, 200, 1280),
+                                   helpers.quick(7, 48, 2040)])
 @pytest.mark.parametrize("pdtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_product(ops, M, N, K, pdtype):
     helpers.skip_in_simulation_if(M * N * K > 1.2e8)
