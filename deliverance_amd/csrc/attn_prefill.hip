@@ -17,6 +17,16 @@
 // Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:458-502.
 // A row's sums run over key tiles in ascending order starting at the aligned tile of its lo: the
 // order depends on the row's position (and window) only.
+//
+// Few workgroups (a prompt of a thousand tokens and a dozen heads gives fewer than the chip has
+// compute units, and the one with the last rows walks all keys alone): the wavefronts of a
+// workgroup then also share out the keys.  RB row blocks of 32 x KP key phases: a round parks KP
+// consecutive tiles in KP LDS buffers, wavefront (row block, phase k) multiplies tile k of the round,
+// and at the end the phases' partial results (maximum, sum of weights, weighted sum) are merged in
+// LDS in the order of the phases.  A tile's phase is (first key / 64) mod KP, whatever the workgroup:
+// a row's sums still depend on its position, the window and KP only; RB x KP is chosen from the
+// step's shape on the host.  Smaller row blocks are for short portions only: every row block of 32
+// reads its keys anew, and on long prompts that traffic, not the longest workgroup, binds.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -25,12 +35,16 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 #define PF_BK 64           // keys per tile
 #define PF_VLD (PF_BK + 8) // padded length of a value row in LDS
 #define PF_BT_MAX 2048      // block-table entries a workgroup keeps in LDS (more are read from memory)
+#define PF_BT_MAX_PHASED 512   // ... where key phases need the LDS for their tiles
+#define PF_PHASED_MAX_WORKGROUPS 256   // 128-row workgroups up to which eight wavefronts (4 x 2) are ahead of four: one a compute unit
 
 // head size / 16; wavefronts (32 query rows each) per workgroup; whether the block table's entries
 // for the workgroup's keys fit its LDS copy (a table entry read from memory in front of a tile's loads
 // makes them wait for it, and for every load still in flight)
-template <int D16, int PF_WAVES, bool BT_LDS>
-__global__ void __launch_bounds__(PF_WAVES * DA_WAVE)
+template <int D16, int RB, int KP, bool BT_LDS>
+// (head sizes up to 64 with key phases and four wavefronts: registers held to 256, so that two
+// workgroups share a compute unit)
+__global__ void __launch_bounds__(RB * KP * DA_WAVE, (KP > 1 && RB * KP == 4 && D16 <= 4) ? 2 : 1)
 attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                     const int* __restrict__ block_table, int max_blocks,
                     const int* __restrict__ q_start, const int* __restrict__ seq_lens, int seq0,
@@ -39,13 +53,22 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   constexpr int D = D16 * 16;
   constexpr int DT = (D + 31) / 32;       // 32-dimension tiles of the output
   constexpr int KLD = D + 8;              // padded length of a key row in LDS
-  constexpr int PF_BQ = PF_WAVES * 32;    // query rows per workgroup
+  constexpr int PF_WAVES = RB * KP;
+  constexpr int PF_BQ = RB * 32;          // query rows per workgroup
   constexpr int THREADS = PF_WAVES * DA_WAVE;
-  constexpr int K_PIECES = PF_BK * (D / 8), V_PIECES = DT * 32 * (PF_BK / 8);   // 16-byte pieces of a tile
+  // one phase: two buffers, a tile is multiplied out of one while the next is parked in the other;
+  // KP phases: the KP tiles of a round
+  constexpr int NB = KP == 1 ? 2 : KP;
+  constexpr int RT = KP == 1 ? 1 : KP;    // tiles that one fetch asks for
+  constexpr int K_PIECES = RT * PF_BK * (D / 8), V_PIECES = RT * DT * 32 * (PF_BK / 8);   // 16-byte pieces of a fetch
   constexpr int NK = (K_PIECES + THREADS - 1) / THREADS, NV = (V_PIECES + THREADS - 1) / THREADS;  // per thread
-  __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][PF_BK * KLD];          // a tile is multiplied out of one
-  __shared__ __attribute__((aligned(16))) bf16_t Vs2[2][DT * 32 * PF_VLD];     // while the next is parked in the other
-  __shared__ int bts[PF_BT_MAX];
+  constexpr int K_TILE = PF_BK * KLD, V_TILE = DT * 32 * PF_VLD;              // elements of a parked tile
+  constexpr int MERGE_FLOATS = (KP - 1) * RB * (DT * 16 + 2) * DA_WAVE;       // the phases' partial results
+  constexpr int TILE_BYTES = NB * (K_TILE + V_TILE) * 2;
+  __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES > MERGE_FLOATS * 4 ? TILE_BYTES : MERGE_FLOATS * 4];
+  bf16_t (*Ks2)[K_TILE] = (bf16_t (*)[K_TILE])smem;
+  bf16_t (*Vs2)[V_TILE] = (bf16_t (*)[V_TILE])(smem + NB * K_TILE * 2);
+  __shared__ int bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];
 
   const int s = seq0 + blockIdx.z, h = blockIdx.y;
   const int row0 = q_start[s], T = q_start[s + 1] - row0;
@@ -57,9 +80,11 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   const int* bt = block_table + (size_t)s * max_blocks;
   const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
   const int col = lane % 32, hf = lane / 32;
+  const int rbi = wave % RB, kp = wave / RB;       // the wavefront's row block and key phase
+  const int wrow = rbi * 32;
 
   // this lane's query row (as a column of Q^T) and its position
-  const int qi = i0 + wave * 32 + col;
+  const int qi = i0 + wrow + col;
   const bool q_ok = qi < T;
   const int pq = past + qi;
   const int q_lo = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
@@ -71,9 +96,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     qf[kd] = __builtin_bit_cast(bf16x8_t, v);
   }
   // the wavefront's rows span positions w_first .. w_last
-  const int w_first = past + i0 + wave * 32;
-  const int w_last_row = (i0 + wave * 32 + 31 < T - 1) ? i0 + wave * 32 + 31 : T - 1;
-  const bool wave_on = i0 + wave * 32 < T;
+  const int w_first = past + i0 + wrow;
+  const int w_last_row = (i0 + wrow + 31 < T - 1) ? i0 + wrow + 31 : T - 1;
+  const bool wave_on = i0 + wrow < T;
   const int w_last = past + w_last_row;
   const int w_lo = (window > 0 && w_first - window + 1 > 0) ? w_first - window + 1 : 0;
   // the workgroup's keys
@@ -107,6 +132,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   const bf16_t* kbase = cache + (long long)hk * page * D;
   const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
   // a tile whose 64 keys all lie in b_lo .. b_last: nothing to clamp, nothing to replace
+  // (a fetch covers RT consecutive tiles: key rows kt .. kt + 64 RT - 1; a value piece is 8 keys of
+  // one dimension of one tile)
+  constexpr int VG = PF_BK / 8, VPT = DT * 32 * VG;       // key groups a tile; value pieces a tile
   auto fetch_fast = [&](uint4* rk, uint4* rv, int kt) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
@@ -117,7 +145,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
-      const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;
+      const int tl = c / VPT, d = (c % VPT) / VG, g = c % VG, key0 = kt + tl * PF_BK + g * 8;
       const int ds = d < D ? d : 0;                      // rows of a padded 32-dimension tile repeat dimension 0
       rv[i] = *(const uint4*)(vbase + page_of(key0 >> lg) * page_elems + ds * page + (key0 & (page - 1)));
     }
@@ -135,7 +163,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
-      const int d = c / (PF_BK / 8), g = c % (PF_BK / 8), key0 = kt + g * 8;   // 8 keys of one dimension
+      const int tl = c / VPT, d = (c % VPT) / VG, g = c % VG, key0 = kt + tl * PF_BK + g * 8;   // 8 keys of one dimension
       const bool ok = d < D && key0 + 7 >= b_lo && key0 <= b_last;
       const int ks = ok ? key0 : (b_last / 8) * 8;
       const int ds = d < D ? d : 0;
@@ -151,21 +179,22 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       rv[i] = v;
     }
   };
+  // (one phase: the tile goes to buffer `buf`; KP phases: tile k of the fetch goes to buffer k)
   auto stash = [&](const uint4* rk, const uint4* rv, int buf) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int c = t + i * THREADS, kr = c / (D / 8), pc = c % (D / 8);
-      if (K_PIECES % THREADS == 0 || c < K_PIECES) *(uint4*)&Ks2[buf][kr * KLD + pc * 8] = rk[i];
+      if (K_PIECES % THREADS == 0 || c < K_PIECES) *(uint4*)&Ks2[buf + kr / PF_BK][(kr % PF_BK) * KLD + pc * 8] = rk[i];
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int c = t + i * THREADS, d = c / (PF_BK / 8), g = c % (PF_BK / 8);
-      if (V_PIECES % THREADS == 0 || c < V_PIECES) *(uint4*)&Vs2[buf][d * PF_VLD + g * 8] = rv[i];
+      const int c = t + i * THREADS, tl = c / VPT, d = (c % VPT) / VG, g = c % VG;
+      if (V_PIECES % THREADS == 0 || c < V_PIECES) *(uint4*)&Vs2[buf + tl][d * PF_VLD + g * 8] = rv[i];
     }
   };
-  const int kt0 = (b_lo / PF_BK) * PF_BK;
+  const int kt0 = (b_lo / (RT * PF_BK)) * (RT * PF_BK);
   fetch(rk0, rv0, kt0);
-  if (kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
+  if (KP == 1 && kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
 
   // the products of one tile, out of LDS buffer `buf`
   auto tile = [&](int kt, int buf) {
@@ -261,6 +290,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   // asked for (two ahead) lies whole inside the workgroup's keys; the last tiles run through the
   // same steps with conditions and the clamping loads.  One barrier a tile: the buffer written now
   // was last read two tiles ago, before the previous barrier.
+  if constexpr (KP == 1) {
   int kt = kt0;
   for (; kt + 4 * PF_BK - 1 <= b_last; kt += 2 * PF_BK) {
     stash(rk0, rv0, 0);
@@ -284,6 +314,48 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     }
     tile(kt, parity);
   }
+  } else {
+    // Key phases: a round parks KP tiles (one register set: the next round's loads fly while this
+    // round's tiles are multiplied), each wavefront multiplies the tile of its phase.  Two barriers a
+    // round: the tiles are parked before anyone reads them and read before they are replaced.
+    for (int kt = kt0; kt <= b_last; kt += KP * PF_BK) {
+      stash(rk0, rv0, 0);
+      lds_barrier();
+      const int nx = kt + KP * PF_BK;
+      if (nx + KP * PF_BK - 1 <= b_last) fetch_fast(rk0, rv0, nx);     // (nx >= b_lo: only the first round starts below it)
+      else if (nx <= b_last) fetch(rk0, rv0, nx);
+      tile(kt + kp * PF_BK, kp);
+      lds_barrier();
+    }
+    // the phases' partial results, merged by phase 0 in the order of the phases
+    float* mg = (float*)smem;
+    constexpr int PER = DT * 16 + 2;
+    if (kp > 0) {
+      float* mine = mg + (size_t)((kp - 1) * RB + rbi) * PER * DA_WAVE + lane;
+#pragma unroll
+      for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mine[(i * 16 + r) * DA_WAVE] = acc_o[i][r];
+      mine[(DT * 16) * DA_WAVE] = m;
+      mine[(DT * 16 + 1) * DA_WAVE] = l;
+    }
+    lds_barrier();
+    if (kp > 0) return;
+#pragma unroll
+    for (int k = 1; k < KP; ++k) {
+      const float* theirs = mg + (size_t)((k - 1) * RB + rbi) * PER * DA_WAVE + lane;
+      const float mk = theirs[(DT * 16) * DA_WAVE], lk = theirs[(DT * 16 + 1) * DA_WAVE];
+      const float m_new = fmaxf(m, mk);
+      const float m_use = m_new != -INFINITY ? m_new : 0.f;
+      const float a0 = __builtin_amdgcn_exp2f(m - m_use), a1 = __builtin_amdgcn_exp2f(mk - m_use);
+      l = l * a0 + lk * a1;
+      m = m_new;
+#pragma unroll
+      for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = acc_o[i][r] * a0 + theirs[(i * 16 + r) * DA_WAVE] * a1;
+    }
+  }
 
   if (q_ok) {
     const float inv = 1.0f / l;
@@ -305,7 +377,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const int* block_table,
                                int max_blocks, const int* q_start, const int* seq_lens, int seq0, int n_seqs,
                                int max_query_len, int Hq, int Hkv, int D, int page, float scale, int window,
-                               void* out, int out_ld, void* stream) {
+                               void* out, int out_ld, int form, void* stream) {
   DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && page > 0 && max_query_len >= 0, "attn_prefill: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_prefill: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attn_prefill: head size %d is not a multiple of 16 up to 256", D);
@@ -318,22 +390,58 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   DA_REQUIRE(n_seqs <= 65535 && Hq <= 65535, "attn_prefill: too many sequences or heads for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
+  // The workgroup's form, row blocks x key phases.  Short portions (after a long past, beside decoded
+  // tokens) have few rows to a sequence and head: 1 x 4 up to 32 rows, 2 x 2 up to 64, so that all four
+  // wavefronts work and share out the keys.  Longer ones take 128 rows a workgroup (smaller row blocks
+  // read the keys more often, and that traffic binds), and 4 x 2, eight wavefronts, while there is no
+  // more than one workgroup a compute unit; else 4 x 1.  Measured on MI355X, head size 64, microseconds
+  // 4x1 / 4x2 / 2x2 / 1x4: 2 x 1,024 rows, 12 heads 23.3 / 19.3 / 23.4 / 34.6; 2,048 rows 40.0 / 31.8 /
+  // 38.9 / 51.7; 8 x 512 rows 19.3 / 23.3 / 26.2 / 42.5; 4 x 64 rows after 900 keys 22.8 / 17.8 / 17.8 /
+  // 16.3; 16 x 2 rows after 1,000 keys 22.8 / 18.5 / 18.3 / 18.0.  Forms with phases need their tiles in LDS at once: head sizes up
+  // to 64 (4 x 2, 1 x 4) or 128 (2 x 2).  The choice reads the step's shape only.
+  // form: 0 leaves the choice to this rule; 41, 42, 22 or 14 fixes it
+  const long per128 = (long)da_ceil_div(max_query_len, 128) * Hq * n_seqs;
+  const int chosen = form ? form
+                     : (D <= 64 && max_query_len <= 32) ? 14
+                     : (D <= 128 && max_query_len <= 64) ? 22
+                     : (D <= 64 && per128 <= PF_PHASED_MAX_WORKGROUPS) ? 42 : 41;
+  DA_REQUIRE(chosen == 41 || (chosen == 22 && D <= 128) || ((chosen == 42 || chosen == 14) && D <= 64),
+             "attn_prefill: form %d with a head size of %d (41 for any; 22 up to 128; 42 and 14 up to 64)", chosen, D);
   // every key a workgroup can see lies within max_blocks pages
-  const bool bt_lds = max_blocks <= PF_BT_MAX;
-#define LAUNCH2(N, W, L)                                                                                  \
-  hipLaunchKernelGGL((attn_prefill_kernel<N, W, L>), dim3(da_ceil_div(max_query_len, 32 * W), Hq, n_seqs), \
-                     dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
+  const bool bt_lds = max_blocks <= (chosen == 41 ? PF_BT_MAX : PF_BT_MAX_PHASED);
+#define LAUNCH2(N, RB, KP, L)                                                                                  \
+  hipLaunchKernelGGL((attn_prefill_kernel<N, RB, KP, L>), dim3(da_ceil_div(max_query_len, 32 * RB), Hq, n_seqs), \
+                     dim3(RB * KP * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
                      max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld)
-#define LAUNCH(N)                      \
-  case N:                              \
-    if (bt_lds) LAUNCH2(N, 4, true);   \
-    else LAUNCH2(N, 4, false);         \
+#define LAUNCH3(N, RB, KP)                \
+  do {                                    \
+    if (bt_lds) LAUNCH2(N, RB, KP, true); \
+    else LAUNCH2(N, RB, KP, false);       \
+  } while (0)
+#define LAUNCH_SMALL(N)                     \
+  case N:                                   \
+    if (chosen == 14) LAUNCH3(N, 1, 4);     \
+    else if (chosen == 22) LAUNCH3(N, 2, 2); \
+    else if (chosen == 42) LAUNCH3(N, 4, 2); \
+    else LAUNCH3(N, 4, 1);                  \
+    break;
+#define LAUNCH_MID(N)                       \
+  case N:                                   \
+    if (chosen == 22) LAUNCH3(N, 2, 2);     \
+    else LAUNCH3(N, 4, 1);                  \
+    break;
+#define LAUNCH(N)                           \
+  case N:                                   \
+    LAUNCH3(N, 4, 1);                       \
     break;
   switch (D / 16) {
-    LAUNCH(1) LAUNCH(2) LAUNCH(3) LAUNCH(4) LAUNCH(5) LAUNCH(6) LAUNCH(7) LAUNCH(8)
+    LAUNCH_SMALL(1) LAUNCH_SMALL(2) LAUNCH_SMALL(3) LAUNCH_SMALL(4) LAUNCH_MID(5) LAUNCH_MID(6) LAUNCH_MID(7) LAUNCH_MID(8)
     LAUNCH(9) LAUNCH(10) LAUNCH(11) LAUNCH(12) LAUNCH(13) LAUNCH(14) LAUNCH(15) LAUNCH(16)
   }
 #undef LAUNCH
+#undef LAUNCH_MID
+#undef LAUNCH_SMALL
+#undef LAUNCH3
 #undef LAUNCH2
   DA_CHECK_LAUNCH("attn_prefill");
   return 0;

@@ -47,6 +47,9 @@ template <int BM, int BN, int OUTMODE>
 constexpr int tile_out_bytes() {
   return BM * (BN + (OUTMODE == 0 ? 8 : 4)) * (OUTMODE == 0 ? 2 : 4);
 }
+// ... and behind it, for a fused q|k|v projection, the tile rows' places in the cache
+template <int BM, int OUTMODE>
+constexpr int tile_slot_bytes() { return OUTMODE == 0 ? BM * 4 : 0; }
 
 template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
 __device__ __forceinline__ void
@@ -123,30 +126,62 @@ tile_epilogue(floatx16 (&acc)[BM / WM / 32][BN / WN / 32], const float (&bias)[B
     }
   }
 
-  // a fused q|k|v projection: the k and v columns also go to the rows' places in the paged cache
+  // A fused q|k|v projection: the k and v columns also go to the rows' places in the paged cache.
+  // Keys are rows there: a piece of 8 columns is a piece of the key's row.  Values are dimension-major
+  // (dimension d of a page's rows side by side): 8 consecutive tile rows of one column are one 16-byte
+  // piece where their places are 8 consecutive rows of one page from a multiple of 8 on (a prompt
+  // portion mostly is), and go entry by entry otherwise.
   if (OUTMODE == 0 && kv.cache) {
-    int pg[NCHK], prow[NCHK];
-#pragma unroll
-    for (int k = 0; k < NCHK; ++k) {
-      const int slot = kv.slot_map[mm[k] < M ? mm[k] : M - 1];
-      pg[k] = slot < 0 ? -1 : slot / kv.page;
-      prow[k] = slot < 0 ? 0 : slot % kv.page;
-    }
+    int* slots = (int*)(smem + tile_out_bytes<BM, BN, OUTMODE>());      // the tile rows' places, -1: none
+    for (int i = t; i < BM; i += THREADS) slots[i] = m0 + i < M ? kv.slot_map[m0 + i] : -1;
+    lds_barrier();
     const bool kwide = (uintptr_t)kv.cache % 16 == 0 && kv.D % 8 == 0 && kv.q_cols % 8 == 0;
+    const int v0 = kv.q_cols + kv.kv_cols;                              // the first value column
 #pragma unroll
     for (int k = 0; k < NCHK; ++k) {
-      if (mm[k] >= M || nn[k] >= N || nn[k] + 8 <= kv.q_cols || pg[k] < 0) continue;
-      const int c2 = nn[k] - kv.q_cols;
-      if (kwide && c2 < kv.kv_cols) {           // eight dimensions of one key: one piece of its row
-        const int h = c2 / kv.D, d = c2 % kv.D;
-        *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg[k], h, prow[k], kv.Hkv, kv.page, kv.D) + d) = val[k];
+      const int slot = slots[mm[k] - m0];
+      if (slot < 0 || nn[k] >= N || nn[k] + 8 <= kv.q_cols || nn[k] >= v0) continue;
+      const int pg = slot / kv.page, prow = slot % kv.page;
+      if (kwide) {                              // eight dimensions of one key: one piece of its row
+        const int c2 = nn[k] - kv.q_cols, h = c2 / kv.D, d = c2 % kv.D;
+        *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg, h, prow, kv.Hkv, kv.page, kv.D) + d) = val[k];
         continue;
       }
       const uint32_t words[4] = {val[k].x, val[k].y, val[k].z, val[k].w};
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        if (nn[k] + e < N && nn[k] + e >= kv.q_cols)
-          kv_scatter_bits(kv, pg[k], prow[k], nn[k] + e, (bf16_t)(words[e / 2] >> (16 * (e % 2))));
+        if (nn[k] + e >= kv.q_cols && nn[k] + e < v0)
+          kv_scatter_bits(kv, pg, prow, nn[k] + e, (bf16_t)(words[e / 2] >> (16 * (e % 2))));
+    }
+    constexpr int NU = (BM / 8) * BN / THREADS;       // (8 rows, column) units a thread; a wavefront's share one row group
+    static_assert((BM / 8) * BN % THREADS == 0 && BN % 64 == 0, "the tile's value units do not split over the threads");
+    const bool vwide = (uintptr_t)kv.cache % 16 == 0 && kv.page % 8 == 0;
+#pragma unroll
+    for (int k = 0; k < NU; ++k) {
+      const int u = t + THREADS * k, g = u / BN, cl = u % BN, n = n0 + cl;
+      if (n < v0 || n >= N) continue;
+      const int cc = n - v0, h = cc / kv.D, d = cc % kv.D;
+      const bf16_t* col = (const bf16_t*)smem + (size_t)(8 * g) * LDT + cl;
+      int sl[8];
+      uint32_t bits[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        sl[e] = slots[8 * g + e];
+        bits[e] = col[e * LDT];
+      }
+      bool run = vwide && sl[0] >= 0 && sl[0] % 8 == 0 && sl[0] % kv.page + 7 < kv.page;
+#pragma unroll
+      for (int e = 1; e < 8; ++e) run = run && sl[e] == sl[0] + e;
+      bf16_t* vb = (bf16_t*)kv.cache;
+      if (run) {
+        const uint4 pk = make_uint4(bits[0] | bits[1] << 16, bits[2] | bits[3] << 16, bits[4] | bits[5] << 16, bits[6] | bits[7] << 16);
+        *(uint4*)(vb + cache_v_base(sl[0] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[0] % kv.page) = pk;
+        continue;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (sl[e] >= 0)
+          vb[cache_v_base(sl[e] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[e] % kv.page] = (bf16_t)bits[e];
     }
   }
 }
@@ -311,7 +346,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
                  Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
   // two buffers of a slab of a and of w; the epilogue parks the tile's results in the same memory
   constexpr int SLAB_BYTES = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16_t);
-  constexpr int OUT_BYTES = tile_out_bytes<BM, BN, OUTMODE>();
+  constexpr int OUT_BYTES = tile_out_bytes<BM, BN, OUTMODE>() + tile_slot_bytes<BM, OUTMODE>();
   __shared__ __attribute__((aligned(16))) char smem[SLAB_BYTES > OUT_BYTES ? SLAB_BYTES : OUT_BYTES];      // shared by the two bodies
   if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);
   else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);

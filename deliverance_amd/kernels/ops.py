@@ -78,7 +78,7 @@ _ARGTYPES = {
     "da_attn_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
     "da_attn_decode": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
     "da_attn_decode_split": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
-    "da_attn_prefill": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_prefill": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP],
     "da_sample": [_VP, _I, _I, _I, _VP, _VP, _VP],
     "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
 }
@@ -432,10 +432,10 @@ def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-# Measured on MI355X (2,048 rows): in the tile kernel's epilogue the cache write doubles the product's
-# time (two-byte stores, scattered for the values); the write kernel after it costs half of that.  For a
-# handful of rows the epilogue saves a kernel.
-KV_EPILOGUE_MAX_ROWS = 64
+# Measured on MI355X (q|k|v of 768 to 1,600 wide, 128 to 2,048 rows): the cache write in the product's
+# epilogue adds 1.3 to 3.4 us where the rows' places are runs of consecutive cache rows (a prompt
+# portion: keys and values both go over in 16-byte pieces), the write kernel after the product 3.7 to
+# 9.2 us; with places in any order the two are level at 2,048 rows and the epilogue is ahead below.
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -446,11 +446,8 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     ``kv_cache`` the k | v columns (from ``q_cols`` on) are also written to the cache rows
     ``slot_map``: in the product's epilogue on the matrix cores, by the write kernel otherwise."""
     if _MODE == "tuned" and _mfma_ok(a, w):
-        if kv_cache is None or a.shape[0] <= KV_EPILOGUE_MAX_ROWS:
-            return linear_mfma(a, w, bias, out, act, accumulate, kv_cache, slot_map, q_cols)
-        linear_mfma(a, w, bias, out, act, accumulate)
-    else:
-        linear_ref(a, w, bias, out, act, accumulate)
+        return linear_mfma(a, w, bias, out, act, accumulate, kv_cache, slot_map, q_cols)
+    linear_ref(a, w, bias, out, act, accumulate)
     if kv_cache is not None:
         _, _, Hkv, _, D = kv_cache.shape
         kv_write(out, q_cols, q_cols + Hkv * D, kv_cache, slot_map, Hkv, D)
@@ -521,9 +518,11 @@ def decode_workspace_floats(n_seqs: int, n_heads: int, head_dim: int, n_splits: 
 def attention_prefill(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,
                       q_start: torch.Tensor, seq_lens: torch.Tensor, seq0: int, n_seqs: int,
                       max_query_len: int, n_heads: int, scale: float, window: Optional[int],
-                      out: torch.Tensor) -> torch.Tensor:
+                      out: torch.Tensor, form: int = 0) -> torch.Tensor:
     """Portions: sequence s (seq0 <= s < seq0 + n_seqs) owns rows q_start[s] .. q_start[s+1]-1 of q
-    and out; its last row sits at position seq_lens[s] - 1."""
+    and out; its last row sits at position seq_lens[s] - 1.  ``form``: a workgroup's row blocks of 32 and
+    the wavefronts that share out a row block's keys, as a two-digit number (41: any head size; 22: up to
+    128; 42 and 14: up to 64); 0 lets the kernel choose from the step's shape."""
     Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_prefill")
     _need(q_start.dtype == torch.int32 and q_start.numel() >= seq0 + n_seqs + 1, "attention_prefill: q_start must be int32 [S+1]")
     _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= seq0 + n_seqs, "attention_prefill: seq_lens must be int32 [S]")
@@ -532,7 +531,7 @@ def attention_prefill(q: torch.Tensor, cache_slot: torch.Tensor, block_table: to
     _check(_lib().da_attn_prefill(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table),
                                         block_table.shape[1], _ptr(q_start), _ptr(seq_lens), seq0, n_seqs,
                                         max_query_len, n_heads, Hkv, D, page, scale,
-                                        int(window or 0), _ptr(out), out.stride(0), _stream()))
+                                        int(window or 0), _ptr(out), out.stride(0), form, _stream()))
     return out
 
 

@@ -312,13 +312,46 @@ def test_attention_prefill_kernel(ops, Hq, Hkv, D, page, window):
     lens = [70, 200, 131, 64, 2, 300, 513]
     new = [70, 9, 131, 2, 2, 129, 260]            # whole prompts, short portions after a long past, tiles' edges
     case = PagedCase(lens=lens, new=new, Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + 2)
-    out = torch.full_like(case.qcat, float("nan"))
     scale = 0.7 / math.sqrt(D)
-    ops.attention_prefill(case.qcat, case.cache, case.bt, case.q_start, case.seq_lens, 0, len(lens), max(new), Hq,
-                          scale, window, out)
-    got = out.double().cpu().numpy()
-    assert np.isfinite(got).all()
-    assert np.abs(got - case.plain(scale, window)).max() < ATT_TOL[torch.bfloat16]
+    want = case.plain(scale, window)
+    # a workgroup's form, row blocks x wavefronts that share out a row block's keys; 0: the kernel's own choice
+    for form in [0, 41] + ([22] if D <= 128 else []) + ([42, 14] if D <= 64 else []):
+        out = torch.full_like(case.qcat, float("nan"))
+        ops.attention_prefill(case.qcat, case.cache, case.bt, case.q_start, case.seq_lens, 0, len(lens), max(new), Hq,
+                              scale, window, out, form=form)
+        got = out.double().cpu().numpy()
+        assert np.isfinite(got).all(), form
+        assert np.abs(got - want).max() < ATT_TOL[torch.bfloat16], form
+    if D > 64:
+        with pytest.raises(ops.KernelError, match="form 14"):
+            ops.attention_prefill(case.qcat, case.cache, case.bt, case.q_start, case.seq_lens, 0, len(lens), max(new), Hq,
+                                  scale, window, out, form=14)
+
+
+@pytest.mark.simt_quick
+@pytest.mark.parametrize("form", [41, 42, 22, 14])
+def test_attention_prefill_finds_a_far_key_in_every_phase(ops, form):
+    """One key among 700 is made to stand out for one query row (key and query scaled up along one
+    direction): the row's output is then that key's value, whichever wavefront's share the key lies in
+    (with 2 or 4 wavefronts to a row block a share is every 2nd or 4th tile of 64 keys) and wherever
+    in its tile."""
+    Hq, Hkv, D, page, n = 2, 2, 64, 16, 700
+    case = PagedCase(lens=[n], new=[n], Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=31)
+    scale = 1.0 / math.sqrt(D)
+    row = n - 1
+    for far in (0, 63, 64, 129, 200, 300, 447, 640, 699):
+        q = case.qcat.clone()
+        cache = case.cache.clone()
+        pg, r = int(case.bt[0, far // page]), far % page
+        direction = torch.zeros(D); direction[far % D] = 30.0
+        for h in range(Hq):
+            q[row, h * D:(h + 1) * D] = direction.to(torch.bfloat16)
+            cache[pg, 0, h, r, :] = direction.to(torch.bfloat16)
+        out = torch.empty_like(q)
+        ops.attention_prefill(q, cache, case.bt, case.q_start, case.seq_lens, 0, 1, n, Hq, scale, None, out, form=form)
+        for h in range(Hq):
+            value = cache[pg, 1, h].reshape(D, page)[:, r].float()          # values lie dimension-major in a page
+            assert (out[row, h * D:(h + 1) * D].float() - value).abs().max() < 2e-2, (far, h)
 
 
 @pytest.mark.simt_quick
@@ -546,7 +579,7 @@ def test_fused_norm_product(ops, M, N, K, pdtype):
         assert (out.double() - ref).abs().max() < tol
 
 
-@pytest.mark.parametrize("M", [helpers.quick(5), helpers.quick(40), 300])
+@pytest.mark.parametrize("M", [helpers.quick(5), helpers.quick(40), helpers.quick(300), 1000])
 def test_product_writes_keys_and_values(ops, M):
     """The skinny (M <= 64) and tile kernels scatter the k | v columns in their epilogue."""
     g = torch.Generator().manual_seed(M)
@@ -558,16 +591,21 @@ def test_product_writes_keys_and_values(ops, M):
     bias = bf(torch.randn(N, generator=g)).to(DEV)
     perm = torch.randperm(n_pages * page, generator=g)[:M].to(torch.int32)
     perm[M // 2] = -1
-    slots = perm.to(DEV)
-    c1 = torch.zeros(n_pages, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
-    c2 = torch.zeros_like(c1)
-    out1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
-    out2 = torch.empty_like(out1)
-    ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D)
-    ops.linear_mfma(a, w, bias, out2)
-    ops.kv_write(out2, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)
-    assert torch.equal(out1, out2)
-    assert torch.equal(c1, c2) and c1.abs().sum() > 0
+    # the places in any order; and as a prompt portion has them: runs of consecutive rows, one from a
+    # multiple of 8 on (values go over in 16-byte runs), one from 3 on, with a token that is not kept
+    runs = torch.cat([torch.arange(16, 16 + M // 2), torch.arange(16 + M // 2 + 19, 16 + M // 2 + 19 + M - M // 2)]).to(torch.int32)
+    runs[M // 4] = -1
+    for order in (perm, runs):
+        slots = order.to(DEV)
+        c1 = torch.zeros(n_pages + 2, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
+        c2 = torch.zeros_like(c1)
+        out1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+        out2 = torch.empty_like(out1)
+        ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D)
+        ops.linear_mfma(a, w, bias, out2)
+        ops.kv_write(out2, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)
+        assert torch.equal(out1, out2)
+        assert torch.equal(c1, c2) and c1.abs().sum() > 0
 
 
 @pytest.mark.simt_quick
