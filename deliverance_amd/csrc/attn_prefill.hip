@@ -189,7 +189,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = t + i * THREADS, tl = c / VPT, d = (c % VPT) / VG, g = c % VG;
-      if (V_PIECES % THREADS == 0 || c < V_PIECES) *(uint4*)&Vs2[buf + tl][d * PF_VLD + g * 8] = rv[i];
+      // Within a block of 16 keys a row keeps them in the order 0-3, 8-11, 4-7, 12-15: the 8 keys a lane
+      // multiplies at once (4hf.., 8+4hf.., as the scores' registers hold them) are then 16 consecutive
+      // bytes, read in one piece and without bank conflicts.
+      if (V_PIECES % THREADS == 0 || c < V_PIECES) {
+        bf16_t* vrow = &Vs2[buf + tl][d * PF_VLD + (g / 2) * 16 + (g % 2) * 4];
+        *(uint2*)vrow = make_uint2(rv[i].x, rv[i].y);
+        *(uint2*)(vrow + 8) = make_uint2(rv[i].z, rv[i].w);
+      }
     }
   };
   const int kt0 = (b_lo / (RT * PF_BK)) * (RT * PF_BK);
@@ -270,16 +277,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] *= alpha;
-      // O^T += V^T . P^T ; the lane's 8 keys of a 16-key block are 4hf..4hf+3 and 8+4hf..8+4hf+3
+      // O^T += V^T . P^T ; the lane's 8 keys of a 16-key block are 4hf..4hf+3 and 8+4hf..8+4hf+3, which
+      // lie side by side in the parked tile
 #pragma unroll
       for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb) {
-            const bf16_t* vr = &Vs[(i * 32 + col) * PF_VLD + ks * 32 + kb * 16 + 4 * hf];
-            const uint2 a0 = *(const uint2*)vr, a1 = *(const uint2*)(vr + 8);
-            const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a0.x, a0.y, a1.x, a1.y));
+            const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Vs[(i * 32 + col) * PF_VLD + ks * 32 + kb * 16 + 8 * hf]);
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[ks][kb], acc_o[i], 0, 0, 0);
           }
     }
