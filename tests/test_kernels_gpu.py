@@ -579,11 +579,11 @@ def test_fused_norm_product(ops, M, N, K, pdtype):
         assert (out.double() - ref).abs().max() < tol
 
 
-@pytest.mark.parametrize("M", [helpers.quick(5), helpers.quick(40), helpers.quick(300), 1000])
+@pytest.mark.parametrize("M", [helpers.quick(5), helpers.quick(40), helpers.quick(300), 1000, 2100])
 def test_product_writes_keys_and_values(ops, M):
     """The skinny (M <= 64) and tile kernels scatter the k | v columns in their epilogue."""
     g = torch.Generator().manual_seed(M)
-    Hq, Hkv, D, page, K = 5, 3, 48, 16, 104
+    Hq, Hkv, D, page, K = 5, 3, 48, 16, (128 if M >= 2000 else 104)      # a K that no slab cuts, too
     N = (Hq + 2 * Hkv) * D
     n_pages = (M + page - 1) // page + 2
     a = bf(torch.randn(M, K, generator=g)).to(DEV)
