@@ -60,16 +60,20 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   const uint4 qraw = *(const uint4*)(q + (size_t)s * q_ld + h * D + (piece_ok ? piece * 8 : 0));
   const int split0 = SPLIT ? (int)blockIdx.y * span : 0;          // the first key of this workgroup's share
   const int c0_guess = split0 + wave * DA_WAVE;
-  int btk0[CPR], btv0[8];
+  // (head sizes above 128 have no registers to spare for them and read the table chunk by chunk)
+  constexpr bool EARLY_BT = CPR <= 16;
+  int btk0[EARLY_BT ? CPR : 1], btv0[EARLY_BT ? 8 : 1];
+  if (EARLY_BT) {
 #pragma unroll
-  for (int i = 0; i < CPR; ++i) {
-    const int pg = (c0_guess + i * G + sub) >> lg;
-    btk0[i] = bt[pg < max_blocks ? pg : max_blocks - 1];
-  }
+    for (int i = 0; i < (EARLY_BT ? CPR : 1); ++i) {
+      const int pg = (c0_guess + i * G + sub) >> lg;
+      btk0[i] = bt[pg < max_blocks ? pg : max_blocks - 1];
+    }
 #pragma unroll
-  for (int g = 0; g < 8; ++g) {
-    const int pg = (c0_guess + g * 8) >> lg;
-    btv0[g] = bt[pg < max_blocks ? pg : max_blocks - 1];
+    for (int g = 0; g < (EARLY_BT ? 8 : 1); ++g) {
+      const int pg = (c0_guess + g * 8) >> lg;
+      btv0[g] = bt[pg < max_blocks ? pg : max_blocks - 1];
+    }
   }
   // the row's position is seq_lens[s] - 1; it sees the keys lo..p (of which this workgroup takes its share)
   const int p_row = seq_lens[s] - 1;
@@ -91,12 +95,29 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     const int last = c0 + DA_WAVE - 1 < p ? c0 + DA_WAVE - 1 : p;
     // the pages of the chunk's keys and value groups: those asked for at the start, or read now
     int btk[CPR], btv[8], bt_safe;
-    if (c0 == c0_guess && first == c0) {                 // the same for the whole wavefront
+    if (EARLY_BT && c0 == c0_guess && first == c0) {     // the same for the whole wavefront
 #pragma unroll
-      for (int i = 0; i < CPR; ++i) btk[i] = btk0[i];
+      for (int i = 0; i < CPR; ++i) btk[i] = btk0[EARLY_BT ? i : 0];
 #pragma unroll
-      for (int g = 0; g < 8; ++g) btv[g] = btv0[g];
+      for (int g = 0; g < 8; ++g) btv[g] = btv0[EARLY_BT ? g : 0];
       bt_safe = __builtin_amdgcn_readfirstlane(btk0[0]); // lane 0 holds the page of key c0
+    } else if (CPR == 32) {
+      // Two keys a load, both in one page (a page has 8 rows at least), and the chunk is the same for
+      // the whole wavefront: the table entries are read by the scalar unit and take no vector registers,
+      // which this head size has none to spare of.
+      const int c0u = __builtin_amdgcn_readfirstlane(c0), fu = __builtin_amdgcn_readfirstlane(first),
+                lu = __builtin_amdgcn_readfirstlane(last);
+      bt_safe = __builtin_amdgcn_readfirstlane(bt[fu >> lg]);
+#pragma unroll
+      for (int i = 0; i < CPR; ++i) {
+        const int k0 = c0u + i * G;                      // the load's first key; G = 2
+        btk[i] = __builtin_amdgcn_readfirstlane(bt[((k0 + G - 1 >= fu && k0 <= lu) ? k0 : fu) >> lg]);
+      }
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const int g0 = c0u + g * 8;
+        btv[g] = __builtin_amdgcn_readfirstlane(bt[((g0 + 7 >= fu && g0 <= lu) ? g0 : fu) >> lg]);
+      }
     } else {
       bt_safe = bt[first >> lg];
 #pragma unroll
@@ -115,14 +136,19 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     for (int i = 0; i < CPR; ++i) {
       const int key = c0 + i * G + sub;
       const bool valid = key >= lo && key <= p;
-      const long long pg = valid ? btk[i] : bt_safe;
+      // (CPR 32: btk[i] is the pair's page, or the page of `first` if neither key is seen, the same for every
+      // lane: the page's address stays with the scalar unit; a lane whose own key is not seen reads some row of it)
+      const long long pg = CPR == 32 ? btk[i] : (valid ? btk[i] : bt_safe);
       const int kk = valid ? key : first;
       kv[i] = *(const uint4*)(kbase + pg * page_elems + (kk & pmask) * D + (piece_ok ? piece * 8 : 0));
     }
     // the chunk's 8 groups of 8 keys (a group never crosses a page) of this lane's first dimension;
     // groups with no seen key read the group of `first` instead and are dropped
+    // (head sizes above 128 hold 128 registers of keys at this point: their values are asked for once the
+    // scores are done, all dimensions at once)
+    constexpr bool EARLY_V = CPR <= 16;
     uint4 vv0[8];
-    {
+    if (EARLY_V) {
       const int d = lane < D ? lane : 0;
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
@@ -172,26 +198,33 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the value loads stay in flight
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    // ---- values: lane owns dimensions lane, lane + 64, ...
+    // ---- values: lane owns dimensions lane, lane + 64, ...; what was not asked for ahead of the scores is
+    // asked for now, every dimension's loads before any is used
+    uint4 vall[DPL][8];
+    if (!EARLY_V) __builtin_amdgcn_sched_barrier(0);    // (not moved up among the scores: the keys' registers are free only now)
 #pragma unroll
     for (int i = 0; i < DPL; ++i) {
-      const int d = lane + i * DA_WAVE;
-      if (DPL > 1 && d >= D) break;
-      float a = acc[i] * alpha;
-      uint4 vv[8];
-      if (i == 0) {
+      if (EARLY_V && i == 0) {
 #pragma unroll
-        for (int g = 0; g < 8; ++g) vv[g] = vv0[g];
+        for (int g = 0; g < 8; ++g) vall[0][g] = vv0[g];
       } else {
+        const int di = lane + i * DA_WAVE, d = di < D ? di : 0;
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
           const int g0 = c0 + g * 8;
           const bool any = g0 + 7 >= first && g0 <= last;
           const int gs = any ? g0 : (first / 8) * 8;
           const long long pg = any ? btv[g] : bt_safe;
-          vv[g] = *(const uint4*)(vbase + pg * page_elems + d * page + (gs & pmask));
+          vall[i][g] = *(const uint4*)(vbase + pg * page_elems + d * page + (gs & pmask));
         }
       }
+    }
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + i * DA_WAVE;
+      if (DPL > 1 && d >= D) break;
+      float a = acc[i] * alpha;
+      const uint4* vv = vall[i];
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
         // Rows outside first..last were never written (or belong to someone else) and may hold anything:
@@ -316,8 +349,8 @@ static int decode_launch(const void* q, int q_ld, const void* cache, const int* 
   if (pieces <= 2) LAUNCH(2);
   else if (pieces <= 4) LAUNCH(4);
   else if (pieces <= 8) LAUNCH(8);
-  else if (pieces <= 16) LAUNCH(16);
-  else LAUNCH(32);
+  else if (pieces <= 16) LAUNCH2(16, 8);
+  else LAUNCH2(32, 8);
 #undef LAUNCH
 #undef LAUNCH2
 #undef LAUNCH3
