@@ -550,6 +550,14 @@ static int launch_skinny(hipStream_t s, const bf16_t* A, int lda, const bf16_t* 
       mt = mb;
       break;
     }
+  // Three or four row tiles take the LDS of a compute unit for one workgroup; with somewhat more
+  // workgroups than compute units a second, mostly empty round then waits for the first.  Two workgroups
+  // of two row tiles share a compute unit and run side by side (GPT-2 1.5B sizes, 48 and 64 rows: 4 and
+  // 2 % of a decode step).
+  if (grid.y == 1 && mt >= 3 && grid.x > 256 && grid.x <= 512) {
+    grid.y = 2;
+    mt = 2;
+  }
   DA_REQUIRE(mt >= 1 && mt <= 4, "gemm_bf16: %d row tiles", mt);
   // steps in flight: 16 to 20 loads of 16 bytes a lane
   if (mt == 1 && M <= 8) DA_SK_GO(1, 16, 4);
