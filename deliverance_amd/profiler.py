@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import time
 from contextlib import contextmanager
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 
 class InferenceProfiler:
@@ -69,13 +69,15 @@ class KernelProfiler:
     MI355X's peaks (8 TB/s of HBM; 2.5 PFLOP/s of bfloat16 matrix products, 157.3 TFLOP/s of
     32-bit arithmetic): the fraction of the roofline that binds that kernel, i.e. the larger of the
     two.  Steps must run kernel by kernel for this (the engine switches recorded graphs off), and
-    the events cost a few microseconds a launch, so the totals are for comparison between kernels,
-    not the engine's speed.  The reference prints per-stage totals in the same place
+    the events cost a few microseconds a launch: what two events with nothing between them measure
+    (the median of 200 pairs, ``overhead_us``) is taken off every launch, and the totals are still for
+    comparison between kernels, not the engine's speed.  The reference prints per-stage totals in the same place
     (core/src/main/java/io/teknek/deliverance/model/InferenceProfiler.java:44-82)."""
     enabled = False
     HBM_BYTES_PER_S = 8.0e12
     PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
     _open: List[tuple] = []          # (name, bytes, flops, precision, start event, end event)
+    overhead_us: Optional[float] = None   # what a pair of events measures with no kernel between them
 
     @classmethod
     def enable(cls) -> None:
@@ -103,16 +105,31 @@ class KernelProfiler:
             cls._open.append((name, float(nbytes), float(flops), precision, a, b))
 
     @classmethod
+    def calibrate(cls) -> float:
+        import torch
+        pairs = []
+        for _ in range(200):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); b.record()
+            pairs.append((a, b))
+        torch.cuda.synchronize()
+        times = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+        cls.overhead_us = times[len(times) // 2]
+        return cls.overhead_us
+
+    @classmethod
     def rows(cls) -> List[dict]:
         """One record per kernel name: calls, total microseconds, bytes, flops, GB/s, TFLOP/s and the
         fraction of the binding roofline."""
         import torch
         torch.cuda.synchronize()
+        if cls.overhead_us is None:
+            cls.calibrate()
         acc: Dict[str, list] = {}
         for name, nb, fl, prec, a, b in cls._open:
             r = acc.setdefault(name, [0, 0.0, 0.0, 0.0, prec])
             r[0] += 1
-            r[1] += a.elapsed_time(b) * 1e3        # microseconds
+            r[1] += max(a.elapsed_time(b) * 1e3 - cls.overhead_us, 0.1)        # microseconds
             r[2] += nb
             r[3] += fl
         out = []
@@ -128,7 +145,7 @@ class KernelProfiler:
     def summary(cls, label: str = "") -> str:
         rows = cls.rows()
         total = sum(r["total_us"] for r in rows) or 1.0
-        lines = [f"kernel summary {label}".rstrip(),
+        lines = [f"kernel summary {label}".rstrip() + f" ({cls.overhead_us:.1f} us of event overhead taken off every launch)",
                  f"{'kernel':28s} {'calls':>7s} {'total_us':>11s} {'mean_us':>9s} {'%time':>6s} {'GB/s':>9s} {'TFLOP/s':>9s} "
                  f"{'bound':>6s} {'%roofline':>9s}"]
         for r in rows:
