@@ -20,6 +20,10 @@
 
 #define DEC_MAX_D 256
 
+// e^x by the hardware's exp2 (two instructions; the library's expf is a dozen, and the merge of 16 wavefronts'
+// partial results takes 16 of them on the one wavefront that everything waits for)
+__device__ __forceinline__ float dec_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
 // Long contexts with few (sequence, head) pairs: the keys are also split over workgroups.  Workgroup
 // (pair, j) takes the keys j * span .. (j + 1) * span - 1 (span a multiple of 64) and leaves its
 // partial result (the weighted sum before the division, the maximum, the sum of weights: D + 2
@@ -190,8 +194,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     const int key = c0 + kidx;
     const bool valid = key >= lo && key <= p;
     const float m_new = fmaxf(m, wave_max(mine));
-    const float e = valid ? expf(mine - m_new) : 0.f;
-    const float alpha = expf(m - m_new);
+    const float e = valid ? dec_exp(mine - m_new) : 0.f;
+    const float alpha = dec_exp(m - m_new);
     l = l * alpha + wave_sum(e);
     m = m_new;
     ps[wave][kidx] = e;
@@ -268,7 +272,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   float f[DEC_WAVES];
 #pragma unroll
   for (int w2 = 0; w2 < DEC_WAVES; ++w2) {
-    f[w2] = part_m[w2] == -INFINITY ? 0.f : expf(part_m[w2] - mm);
+    f[w2] = part_m[w2] == -INFINITY ? 0.f : dec_exp(part_m[w2] - mm);
     ll += part_l[w2] * f[w2];
   }
   if (SPLIT) {
@@ -303,14 +307,14 @@ attn_decode_merge_kernel(const float* __restrict__ partial, int n_splits, int Hq
   float ll = 0.f;
   for (int j = 0; j < n_splits; ++j) {
     const float mj = mine[(size_t)j * (D + 2) + D];
-    ll += mine[(size_t)j * (D + 2) + D + 1] * (mj == -INFINITY ? 0.f : expf(mj - mm));
+    ll += mine[(size_t)j * (D + 2) + D + 1] * (mj == -INFINITY ? 0.f : dec_exp(mj - mm));
   }
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float o = 0.f;
     for (int j = 0; j < n_splits; ++j) {
       const float mj = mine[(size_t)j * (D + 2) + D];
-      o += mine[(size_t)j * (D + 2) + d] * (mj == -INFINITY ? 0.f : expf(mj - mm));
+      o += mine[(size_t)j * (D + 2) + d] * (mj == -INFINITY ? 0.f : dec_exp(mj - mm));
     }
     out[(size_t)s * out_ld + h * D + d] = f32_to_bf16(o * inv);
   }
