@@ -150,6 +150,19 @@ def test_gemm_matrix_cores(ops, M, N, K):
         assert (out - ref).abs().max() < tol, (act, acc, bias, od)
 
 
+@pytest.mark.parametrize("M,N,K", [(1600, 2000, 200), (1555, 1999, 320), (2048, 1600, 1600)])
+def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
+    """192 to 256 tiles of 128 x 128: the form with four slabs in flight (a K that a slab cuts, a K of
+    five whole slabs, GPT-2 1.5B's out-proj)."""
+    helpers.skip_in_simulation_if(True)
+    g = torch.Generator().manual_seed(M + N + K)
+    for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
+                               (None, True, True, torch.float32), (None, False, False, torch.float32)):
+        out, ref = _gemm_case(ops, ops.linear_mfma, M, N, K, torch.bfloat16, act, acc, bias, od, g)
+        tol = (1e-2 if od == torch.bfloat16 else 1e-4) * max(1.0, ref.abs().max().item())
+        assert (out - ref).abs().max() < tol, (act, acc, bias, od)
+
+
 @pytest.mark.simt_quick
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """A row's result is the same, bit for bit, whatever other rows share the call, as long as the call
