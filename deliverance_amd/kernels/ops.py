@@ -132,7 +132,8 @@ def _dev(*ts):
 
 
 def _rows_2d(t: torch.Tensor, name: str):
-    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with a contiguous last dimension")
+    if not (t.dim() == 2 and t.stride(1) == 1):
+        raise KernelError(f"{name} must be 2-D with a contiguous last dimension")
 
 
 # ------------------------------------------------------------------------------- embedding
@@ -209,11 +210,14 @@ def linear_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], o
     _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
     M, K = a.shape
     N = w.shape[0]
-    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
-    _need(out.shape[0] == M and out.shape[1] == N, f"linear: out is {list(out.shape)}, expected [{M},{N}]")
+    if not (w.shape[1] == K):
+        raise KernelError(f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    if not (out.shape[0] == M and out.shape[1] == N):
+        raise KernelError(f"linear: out is {list(out.shape)}, expected [{M},{N}]")
     _need(a.dtype == w.dtype, "linear: a and w must share a dtype")
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
-    _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
     with _timed("linear_ref", _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K, "fp32"):
         _check(_lib().da_gemm_ref(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _dt(a), _ptr(bias),
@@ -347,7 +351,8 @@ def _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, name):
     _, _, Hkv, page, D = kv_cache.shape
     _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= n_rows,
           f"{name}: slot_map must be int32 [rows]")
-    _need(q_cols + 2 * Hkv * D == N, f"{name}: q|k|v columns do not add up to N")
+    if not (q_cols + 2 * Hkv * D == N):
+        raise KernelError(f"{name}: q|k|v columns do not add up to N")
     return _ptr(kv_cache), _ptr(slot_map), q_cols, Hkv * D, Hkv, D, page
 
 
@@ -361,15 +366,21 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     M, K = a.shape
     N = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_mfma: a and w must be bfloat16")
-    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
-    _need(out.shape[0] == M and out.shape[1] == N, f"linear: out is {list(out.shape)}, expected [{M},{N}]")
+    if not (w.shape[1] == K):
+        raise KernelError(f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    if not (out.shape[0] == M and out.shape[1] == N):
+        raise KernelError(f"linear: out is {list(out.shape)}, expected [{M},{N}]")
     _need(bias is None or bias.numel() == N, "linear: bias length differs from N")
-    _need(act in ACTIVATIONS, f"linear: unknown activation {act!r}")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"linear: unknown activation {act!r}")
     _need(not accumulate or out.dtype == torch.float32, "linear: accumulation needs a float32 output")
     _need(kv_cache is None or not accumulate, "linear: a cache scatter goes with a plain store")
     kvp = _kv_args(kv_cache, slot_map, q_cols, M, N, out, "linear_mfma")
-    name = "product_skinny" if (M <= 32 or (M <= 64 and N <= 8192)) else "product_tile"
-    with _timed(name, _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K):
+    timing = _NO_TIMING
+    if KernelProfiler.enabled:           # (the cost model is worked out only when someone reads it)
+        name = "product_skinny" if (M <= 32 or (M <= 64 and N <= 8192)) else "product_tile"
+        timing = _timed(name, _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K)
+    with timing:
         _check(_lib().da_gemm_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
                                    _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
                                    _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp, _stream()))
@@ -415,7 +426,8 @@ def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_w
     else:
         _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "linear_ln: rows must be int32")
     _need(bias is None or bias.numel() == N, "linear_ln: bias length differs from N")
-    _need(act in ACTIVATIONS, f"linear_ln: unknown activation {act!r}")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"linear_ln: unknown activation {act!r}")
     kvp = _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, "linear_ln")
     with _timed("norm_product_fused", n_rows * K * 4 + _nbytes(w, bias, norm_weight, norm_bias) + n_rows * N * out.element_size(),
                 2 * n_rows * N * K):
@@ -458,8 +470,10 @@ def _attn_common(q, cache_slot, block_table, n_heads, out, name):
     _dev(q, cache_slot, block_table, out)
     _rows_2d(q, "q"); _rows_2d(out, "out")
     P, two, Hkv, page, D = cache_slot.shape
-    _need(cache_slot.is_contiguous() and two == 2, f"{name}: cache slot must be contiguous [pages,2,Hkv,page,D]")
-    _need(q.shape[1] == n_heads * D and out.shape[1] == n_heads * D, f"{name}: q/out must be [rows, Hq*D]")
+    if not (cache_slot.is_contiguous() and two == 2):
+        raise KernelError(f"{name}: cache slot must be contiguous [pages,2,Hkv,page,D]")
+    if not (q.shape[1] == n_heads * D and out.shape[1] == n_heads * D):
+        raise KernelError(f"{name}: q/out must be [rows, Hq*D]")
     _need(q.dtype == torch.bfloat16 and cache_slot.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
           f"{name}: q, cache and out must be bfloat16")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
