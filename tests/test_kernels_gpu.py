@@ -164,6 +164,28 @@ def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
 
 
 @pytest.mark.simt_quick
+@pytest.mark.parametrize("M", [20, 200])
+def test_gemm_into_rows_longer_than_the_result(ops, M):
+    """The output's rows are longer than N (a view of a wider matrix): the tile kernel stores whole
+    16-byte pieces up to the last one that N cuts, which goes out entry by entry; what lies behind
+    column N is not touched, with a store, a 32-bit store and +=."""
+    g = torch.Generator().manual_seed(M)
+    N, K, LD = 1030, 96, 1040
+    a = bf(torch.randn(M, K, generator=g) * 0.5).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.2).to(DEV)
+    b = bf(torch.randn(N, generator=g)).to(DEV)
+    ref = a.double() @ w.double().t() + b.double()
+    for od, acc in ((torch.bfloat16, False), (torch.float32, False), (torch.float32, True)):
+        big = torch.full((M, LD), 7.0, device=DEV, dtype=od)
+        out = big[:, :N]
+        ops.linear_mfma(a, w, b, out, None, acc)
+        want = ref + (7.0 if acc else 0.0)
+        tol = (1e-2 if od == torch.bfloat16 else 1e-4) * max(1.0, want.abs().max().item())
+        assert (out.double() - want).abs().max() < tol, (od, acc)
+        assert torch.equal(big[:, N:], torch.full((M, LD - N), 7.0, device=DEV, dtype=od)), (od, acc)
+
+
+@pytest.mark.simt_quick
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """A row's result is the same, bit for bit, whatever other rows share the call, as long as the call
     takes the same kernel form (block tiles; 16x16x32 products up to 64 rows; 4x4x4 products up to 4
