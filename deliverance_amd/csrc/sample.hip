@@ -185,18 +185,19 @@ sample_kernel(const float* __restrict__ logits, int ldl, int V, const SampleRow*
   const SampleRow sp = params[r];
   const float* row = logits + (size_t)r * ldl;
 
-  // the largest entry (the lowest index among equals): eight loads in flight per thread, from clamped
-  // places, so that the vocabulary is crossed in a few memory round trips
+  // the largest entry (the lowest index among equals): ARGMAX_LOADS loads in flight per thread, from
+  // clamped places, so that a vocabulary of 50,000 is crossed in two memory round trips
+  constexpr int ARGMAX_LOADS = 25;
   float best = -INFINITY; int besti = -1;
-  for (int i0 = threadIdx.x; i0 < V; i0 += 8 * SAMPLE_THREADS) {
-    float v[8];
+  for (int i0 = threadIdx.x; i0 < V; i0 += ARGMAX_LOADS * SAMPLE_THREADS) {
+    float v[ARGMAX_LOADS];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < ARGMAX_LOADS; ++u) {
       const int i = i0 + u * SAMPLE_THREADS;
       v[u] = row[i < V ? i : V - 1];
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < ARGMAX_LOADS; ++u) {
       const int i = i0 + u * SAMPLE_THREADS;
       if (i < V && (besti < 0 || v[u] > best)) { best = v[u]; besti = i; }
     }
