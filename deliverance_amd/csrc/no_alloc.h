@@ -21,6 +21,8 @@
 
 #define DA_DECODE_STATIC_SCRATCH_BYTES (8 << 20)
 
+// One stream at a time per GPU: two calls whose kernels may overlap on one GPU (two streams, two host
+// threads, two engines of one process) race on that GPU's one buffer, and nothing detects it.
 extern "C" int da_attn_decode_split_static(const void* q, int q_ld, const void* cache, const int* block_table,
                                            int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D,
                                            int page, float scale, int window, void* out, int out_ld, int n_splits,

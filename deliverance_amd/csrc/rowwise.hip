@@ -99,6 +99,72 @@ extern "C" int da_take_tokens(int* tokens, const int* src, const int* sampled, i
 }
 
 // ------------------------------------------------------------------------------------------
+// Zeros over a buffer of whole 4-byte words (a kernel, so that a recorded step holds no memset node).
+// ------------------------------------------------------------------------------------------
+__global__ void fill_zero_kernel(uint32_t* __restrict__ p, long n_words) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
+}
+
+extern "C" int da_fill_zero(void* p, long n_bytes, void* stream) {
+  DA_REQUIRE(n_bytes >= 0 && n_bytes % 4 == 0 && (uintptr_t)p % 4 == 0, "fill_zero: %ld bytes are not whole words", n_bytes);
+  if (n_bytes == 0) return 0;
+  const long words = n_bytes / 4;
+  const int blocks = (int)(words / 256 < 1 ? 1 : (words / 256 > 2048 ? 2048 : words / 256));
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t*)p, words);
+  DA_CHECK_LAUNCH("fill_zero");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Fixed-size state of the step's sequences, as rows of 4-byte words (any dtype).
+//   gather:  out[n, :] = state[slot[seq_of_token[n]], :]   (zeros where the sequence has no slot: a padding row)
+//   scatter: state[slot[s], :] = rows[q_start[s+1] - 1, :] for every sequence s that has a slot and brings rows
+// A mixer with state reads the first before it walks its rows and calls the second with what each row
+// leaves behind: the state of a portion's last row is the request's state after the step.
+// ------------------------------------------------------------------------------------------
+__global__ void state_gather_kernel(const uint32_t* __restrict__ state, const int* __restrict__ slots,
+                                    const int* __restrict__ seq_of_token, uint32_t* __restrict__ out,
+                                    int n_slots, int words) {
+  const int n = blockIdx.x;
+  const int slot = slots[seq_of_token[n]];
+  const bool has = slot >= 0 && slot < n_slots;
+  for (int i = threadIdx.x; i < words; i += blockDim.x)
+    out[(size_t)n * words + i] = has ? state[(size_t)slot * words + i] : 0u;
+}
+
+__global__ void state_scatter_kernel(uint32_t* __restrict__ state, const int* __restrict__ slots,
+                                     const int* __restrict__ q_start, const uint32_t* __restrict__ rows,
+                                     int n_slots, int words) {
+  const int s = blockIdx.x;
+  const int slot = slots[s], first = q_start[s], last = q_start[s + 1] - 1;
+  if (slot < 0 || slot >= n_slots || last < first) return;
+  for (int i = threadIdx.x; i < words; i += blockDim.x) state[(size_t)slot * words + i] = rows[(size_t)last * words + i];
+}
+
+extern "C" int da_state_gather(const void* state, const int* slots, const int* seq_of_token, void* out, int N,
+                               int n_slots, int row_bytes, void* stream) {
+  DA_REQUIRE(N >= 0 && n_slots > 0 && row_bytes > 0 && row_bytes % 4 == 0, "state_gather: bad sizes (N=%d, %d slots, rows of %d bytes)",
+             N, n_slots, row_bytes);
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(state_gather_kernel, dim3(N), dim3(row_bytes / 4 >= 256 ? 256 : 64), 0, (hipStream_t)stream,
+                     (const uint32_t*)state, slots, seq_of_token, (uint32_t*)out, n_slots, row_bytes / 4);
+  DA_CHECK_LAUNCH("state_gather");
+  return 0;
+}
+
+extern "C" int da_state_scatter(void* state, const int* slots, const int* q_start, const void* rows, int S,
+                                int n_slots, int row_bytes, void* stream) {
+  DA_REQUIRE(S >= 0 && n_slots > 0 && row_bytes > 0 && row_bytes % 4 == 0, "state_scatter: bad sizes (S=%d, %d slots, rows of %d bytes)",
+             S, n_slots, row_bytes);
+  if (S == 0) return 0;
+  hipLaunchKernelGGL(state_scatter_kernel, dim3(S), dim3(row_bytes / 4 >= 256 ? 256 : 64), 0, (hipStream_t)stream,
+                     (uint32_t*)state, slots, q_start, (const uint32_t*)rows, n_slots, row_bytes / 4);
+  DA_CHECK_LAUNCH("state_scatter");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // LayerNorm over rows of 32-bit x; one wave per row; mean and centred variance in 32-bit.
 //   y = (x - mean) / sqrt(var + eps) * w + b        (var biased, eps inside the root)
 // Reference: core/src/main/java/io/teknek/deliverance/generator/LayerNorm.java:127-150

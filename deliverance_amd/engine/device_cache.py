@@ -27,12 +27,14 @@ class DeviceCache:
         self.page_size = check_page_size(page_size)
         by_shape: Dict[tuple, List[int]] = {}
         state_specs: List[StateSpec] = []
+        state_needs: Dict[int, StateNeed] = {}
         for slot in sorted(needs):
             need = needs[slot]
             if isinstance(need, KVNeed):
                 by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window), []).append(slot)
             elif isinstance(need, StateNeed):
                 state_specs.append(StateSpec(slot, need.elems))
+                state_needs[slot] = need
             else:
                 raise TypeError(f"cache slot {slot}: unknown kind of need {need!r}")
         self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w), slots in by_shape.items()]
@@ -52,8 +54,9 @@ class DeviceCache:
                 self.group_of_slot[slot] = g
         self.state: Dict[int, torch.Tensor] = {}
         n_slots = n_state_slots if state_specs else 0
-        for s in state_specs:
-            self.state[s.slot] = torch.zeros((n_slots, s.elems), dtype=torch.float32, device=self.device)
+        for s in state_specs:          # [state slots, *shape] in the dtype the mixer asked for
+            need = state_needs[s.slot]
+            self.state[s.slot] = torch.zeros((n_slots, *need.row_shape), dtype=need.dtype, device=self.device)
         self.manager = CacheManager(self.groups, page_size, [self.n_pages] * len(self.groups),
                                     state_specs, n_slots)
         if poison_freed:
@@ -75,8 +78,18 @@ class DeviceCache:
         el = torch.empty((), dtype=self.dtype).element_size()
         return sum(len(g.slots) * 2 * g.n_kv_heads * g.head_dim * el for g in self.groups)
 
+    def state_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.state.values())
+
     @staticmethod
-    def tokens_for_budget(needs: Dict[int, object], dtype: torch.dtype, budget_bytes: int) -> int:
+    def state_bytes_for(needs: Dict[int, object], n_state_slots: int) -> int:
+        """What the fixed-size state of ``n_state_slots`` requests takes."""
+        return n_state_slots * sum(n.nbytes for n in needs.values() if isinstance(n, StateNeed))
+
+    @staticmethod
+    def tokens_for_budget(needs: Dict[int, object], dtype: torch.dtype, budget_bytes: int, n_state_slots: int = 0) -> int:
+        """How many tokens' keys and values fit into ``budget_bytes`` once the state slots are paid for."""
         el = torch.empty((), dtype=dtype).element_size()
         per_token = sum(2 * n.n_kv_heads * n.head_dim * el for n in needs.values() if isinstance(n, KVNeed))
-        return max(0, budget_bytes // max(per_token, 1))
+        left = budget_bytes - DeviceCache.state_bytes_for(needs, n_state_slots)
+        return max(0, left // max(per_token, 1))

@@ -68,12 +68,12 @@ class CausalLanguageModel:
         self.engine_config = engine_config
         needs = model.cache_needs()
         tokens = engine_config.max_cached_tokens
+        n_slots = engine_config.state_slots if engine_config.state_slots is not None else engine_config.max_num_seqs
         if tokens is None:
             free, _ = torch.cuda.mem_get_info(model.device)
-            tokens = DeviceCache.tokens_for_budget(needs, model.dtype, int(free * 0.5))
+            tokens = DeviceCache.tokens_for_budget(needs, model.dtype, int(free * 0.5), n_slots)
             tokens = min(tokens, engine_config.max_num_seqs * model.config.max_positions)
             tokens = max(tokens, engine_config.page_size)
-        n_slots = engine_config.state_slots if engine_config.state_slots is not None else engine_config.max_num_seqs
         self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots,
                                  poison_freed=engine_config.poison_freed_pages)
         self.runner = StepRunner(model, self.cache, use_graphs=engine_config.use_graphs,
@@ -127,7 +127,7 @@ class CausalLanguageModel:
     def set_layer_debug_hook(self, hook: Optional[Callable]) -> None:
         """``hook(layer, stage, tensor)`` receives copies of named intermediates of every step (layer -1,
         "input": the embedding; per layer "query_projection", "key_projection", "value_projection",
-        "attention_value", "post_attention_residual", "post_ff_residual", "layer_output"), as the
+        "attention_value", "attention_output", "post_attention_residual", "post_ff_residual", "layer_output"), as the
         reference's ``setLayerDebugHook`` does (core/.../model/AbstractModel.java:122-128,505-515,1100-1107).
         While a hook is set, steps run kernel by kernel (no recorded graphs) and slowly."""
         self.runner.debug_hook = hook

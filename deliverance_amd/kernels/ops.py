@@ -15,6 +15,7 @@ from . import build
 from ..profiler import KernelProfiler
 
 F32, BF16 = 0, 1
+MAX_HEAD_DIM = 256          # what the plain attention kernel takes; the matrix-core kernels: multiples of 16 up to it
 ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4}
 
 
@@ -69,6 +70,9 @@ _ARGTYPES = {
     "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _F, _VP],
     "da_copy_rows": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_take_tokens": [_VP, _VP, _VP, _I, _I, _I, _VP],
+    "da_fill_zero": [_VP, ctypes.c_long, _VP],
+    "da_state_gather": [_VP, _VP, _VP, _VP, _I, _I, _I, _VP],
+    "da_state_scatter": [_VP, _VP, _VP, _VP, _I, _I, _I, _VP],
     "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
     "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
@@ -179,6 +183,50 @@ def take_tokens(tokens: torch.Tensor, src: torch.Tensor, sampled: torch.Tensor, 
     _check(_lib().da_take_tokens(_ptr(tokens), _ptr(src), _ptr(sampled), tokens.numel(), sampled.numel(), int(vocab),
                                  _stream()))
     return tokens
+
+
+def fill_zero(t: torch.Tensor) -> torch.Tensor:
+    """Zeros over a contiguous tensor of whole 4-byte words, by a kernel of the engine's own (a recorded
+    step then holds no memset node)."""
+    _dev(t)
+    _need(t.is_contiguous() and (t.numel() * t.element_size()) % 4 == 0, "fill_zero: a contiguous tensor of whole words")
+    _check(_lib().da_fill_zero(_ptr(t), t.numel() * t.element_size(), _stream()))
+    return t
+
+
+def _state_rows(state: torch.Tensor, rows: torch.Tensor, name: str) -> int:
+    _need(state.is_contiguous() and rows.is_contiguous() and state.dtype == rows.dtype and state.dim() >= 2,
+          f"{name}: state [slots, ...] and rows [N, ...] must be contiguous and of one dtype")
+    row_bytes = state[0].numel() * state.element_size()
+    _need(rows.dim() >= 1 and rows.numel() == rows.shape[0] * state[0].numel() and row_bytes % 4 == 0,
+          f"{name}: a row of the state is {state[0].numel()} entries ({row_bytes} bytes, whole words)")
+    return row_bytes
+
+
+def state_gather(state: torch.Tensor, state_slots: torch.Tensor, seq_of_token: torch.Tensor,
+                 out: torch.Tensor) -> torch.Tensor:
+    """out[n] = state[state_slots[seq_of_token[n]]]: every row of the step gets its sequence's state (zeros
+    for a sequence without a slot, i.e. a padding row of a fixed-shape step)."""
+    _dev(state, state_slots, seq_of_token, out)
+    row_bytes = _state_rows(state, out, "state_gather")
+    N = out.shape[0]
+    _need(state_slots.dtype == torch.int32 and seq_of_token.dtype == torch.int32 and seq_of_token.numel() >= N,
+          "state_gather: slots and sequence ids must be int32, one id a row")
+    _check(_lib().da_state_gather(_ptr(state), _ptr(state_slots), _ptr(seq_of_token), _ptr(out), N, state.shape[0],
+                                  row_bytes, _stream()))
+    return out
+
+
+def state_scatter(state: torch.Tensor, state_slots: torch.Tensor, q_start: torch.Tensor, rows: torch.Tensor,
+                  n_seqs: int) -> None:
+    """state[state_slots[s]] = rows[q_start[s + 1] - 1] for every sequence s with a slot: what the last row
+    of a sequence's portion leaves is the request's state after the step."""
+    _dev(state, state_slots, q_start, rows)
+    row_bytes = _state_rows(state, rows, "state_scatter")
+    _need(state_slots.dtype == torch.int32 and q_start.dtype == torch.int32 and state_slots.numel() >= n_seqs
+          and q_start.numel() >= n_seqs + 1, "state_scatter: slots [S] and q_start [S+1] must be int32")
+    _check(_lib().da_state_scatter(_ptr(state), _ptr(state_slots), _ptr(q_start), _ptr(rows), n_seqs, state.shape[0],
+                                   row_bytes, _stream()))
 
 
 # ------------------------------------------------------------------------------- norms
@@ -553,7 +601,8 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
                     scale: float, window: Optional[int], out: torch.Tensor) -> torch.Tensor:
     """Attention of every row of the step over its sequence's pages.  In bfloat16 the one-token
     sequences (the first ``ctx.n_decode``) go to the decode kernel and the portions to the
-    prefill kernel; 32-bit and the reference mode use the plain kernel for all rows."""
+    prefill kernel; 32-bit, the reference mode and head sizes that are no multiple of 16 (which the
+    matrix-core kernels do not take) use the plain kernel for all rows."""
     bt = ctx.block_tables[group]
     Hkv, page, D = cache_slot.shape[2], cache_slot.shape[3], cache_slot.shape[4]
     el = cache_slot.element_size()
@@ -575,7 +624,7 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
             pairs += sum(min(n - t + i + 1, window or n) for i in range(t)) if t > 1 else min(n, window or n)
         return keys * 2 * Hkv * D * el + 2 * rows * n_heads * D * el, 4 * pairs * n_heads * D
 
-    if _MODE == "tuned" and q.dtype == torch.bfloat16:
+    if _MODE == "tuned" and q.dtype == torch.bfloat16 and D % 16 == 0 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0:
         if nd:
             n_splits = decode_splits(nd, n_heads, bt.shape[1], page)
             ws = None

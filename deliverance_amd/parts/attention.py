@@ -23,8 +23,10 @@ class CausalSelfAttention(Mixer):
         self.n_heads, self.n_kv_heads, self.head_dim = spec.n_heads, spec.n_kv_heads, spec.head_dim
         if self.n_heads % self.n_kv_heads != 0:
             raise ValueError(f"{self.n_heads} query heads are not a multiple of {self.n_kv_heads} key heads")
-        if self.head_dim % 16 != 0 or self.head_dim > 256:
-            raise ValueError(f"head size {self.head_dim} is not a multiple of 16 up to 256")
+        # Any head size up to 256 runs: multiples of 16 on the matrix-core attention kernels in bfloat16,
+        # the others (and everything in 32-bit) on the plain attention kernel.
+        if not (1 <= self.head_dim <= ops.MAX_HEAD_DIM):
+            raise ValueError(f"head size {self.head_dim} is outside 1..{ops.MAX_HEAD_DIM}")
         self.q_cols = self.n_heads * self.head_dim
         self.kv_cols = self.n_kv_heads * self.head_dim
         self.qkv_cols = self.q_cols + 2 * self.kv_cols
@@ -89,6 +91,9 @@ class CausalSelfAttention(Mixer):
             ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
             ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:])
             ctx.emit(call.layer, "attention_value", o)
+            # the output projection before its bias (CausalSelfAttention.java:406), worked out once more for the hook
+            ctx.emit(call.layer, "attention_output",
+                     ops.linear(o, self.out_weight, None, ctx.buf("attn_proj_debug", N, x.shape[1], torch.float32)))
         ops.linear(o, self.out_weight, self.out_bias, x, accumulate=True)
 
 

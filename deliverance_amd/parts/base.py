@@ -7,12 +7,17 @@ a new mixer, feed-forward, norm or position encoding is added by registering a b
 
 Interfaces (shapes: N tokens of the step, E model width):
 
-* ``Norm.forward(ctx, x, rows=None) -> h``: x is the 32-bit residual stream [N, E]; h is
-  in the compute dtype, [N, E] or, with ``rows`` (int32 row indices), [len(rows), E].
+* ``Norm.forward(ctx, x, rows=None, out_dtype=None) -> h``: x is the 32-bit residual stream [N, E];
+  h is in the compute dtype (or ``out_dtype``), [N, E] or, with ``rows`` (int32 row indices),
+  [len(rows), E].
 * ``Mixer.forward(ctx, h, x, call) -> None``: reads h, *adds* its result to x in place
   (32-bit).  ``call`` is the run-order entry (cache slot, write flag).
   ``Mixer.cache_need()`` says what the mixer keeps between steps: a ``KVNeed`` (pages of keys
-  and values), a ``StateNeed`` (fixed-size state in a slot per request) or None.
+  and values), a ``StateNeed`` (fixed-size state in a slot per request) or None.  A mixer with
+  state finds everything about the step's rows on the device (``ctx.seq_of_token``,
+  ``ctx.positions``, ``ctx.q_start``, ``ctx.state_slots``); ``ops.state_gather`` hands every row
+  its sequence's state and ``ops.state_scatter`` keeps the state that each portion's last row
+  leaves.  One that reads these only (never the ``*_host`` lists) may set ``graph_safe``.
 * ``FeedForward.forward(ctx, h, x) -> None``: reads h, adds its result to x in place.
 * ``PositionEncoding``: ``embed_table()`` returns a [P, E] table added to token embeddings
   (or None); ``apply_qk(ctx, qkv, ...)`` may rotate queries and keys in place (default: none).
@@ -23,7 +28,7 @@ The reference wires the same roles through constructor arguments of one block cl
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Callable, Dict, List, Optional
+from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
 
@@ -37,7 +42,30 @@ class KVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    elems: int          # 32-bit floats per request
+    """Fixed-size state of one request: ``elems`` entries of ``dtype``, as one row, or in ``shape`` (whose
+    product is ``elems``).  The cache keeps a tensor ``[state slots, *shape]`` of that dtype for it and
+    counts its bytes in the memory it plans with."""
+    elems: int
+    dtype: torch.dtype = torch.float32
+    shape: Optional[Tuple[int, ...]] = None
+
+    def __post_init__(self):
+        if self.elems <= 0:
+            raise ValueError(f"a state of {self.elems} entries")
+        if self.shape is not None:
+            n = 1
+            for d in self.shape:
+                n *= int(d)
+            if n != self.elems:
+                raise ValueError(f"state shape {tuple(self.shape)} does not hold {self.elems} entries")
+
+    @property
+    def row_shape(self) -> Tuple[int, ...]:
+        return tuple(self.shape) if self.shape is not None else (self.elems,)
+
+    @property
+    def nbytes(self) -> int:
+        return self.elems * torch.empty((), dtype=self.dtype).element_size()
 
 
 class StepContext:
@@ -104,7 +132,8 @@ class Arena:
 
 class Norm:
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
-                n_rows: Optional[int] = None, out_name: str = "norm") -> torch.Tensor:
+                n_rows: Optional[int] = None, out_name: str = "norm",
+                out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         raise NotImplementedError
 
     def fusable_params(self):

@@ -34,19 +34,19 @@ class Block:
     @staticmethod
     def _part(ctx, x, pre, post, run, run_normed):
         """One part of the block.  Parts add into the tensor they are given.  Without a norm behind
-        the part that tensor is the residual stream; with one, the part adds into a zeroed buffer
-        of its own, whose norm is then added to the stream."""
+        the part that tensor is the residual stream; with one, the part adds into a buffer of its
+        own (cleared by a fill kernel of the engine's, so that a recorded step holds no memset), whose
+        norm, kept in 32-bit, is then added to the stream."""
         target = x
         if post is not None:
-            target = ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32)
-            target.zero_()
+            target = ops.fill_zero(ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32))
         # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
         # of it itself (fused into its first product) and returns True, or returns False to
         # decline this step.  That needs the part's input and the tensor it adds into to be the same.
         if not (post is None and pre is not None and run_normed is not None and run_normed(pre)):
             run(Block._normed(ctx, x, pre), target)
         if post is not None:
-            ops.copy_rows(post.forward(ctx, target, out_name="post_norm"), x, accumulate=True)
+            ops.copy_rows(post.forward(ctx, target, out_name="post_norm", out_dtype=torch.float32), x, accumulate=True)
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
         fused = getattr(self.mixer, "forward_normed", None)

@@ -20,9 +20,10 @@ class LayerNorm(Norm):
             raise ValueError(f"LayerNorm gain has {self.weight.numel()} entries for width {self.width}")
 
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
-                n_rows: Optional[int] = None, out_name: str = "norm") -> torch.Tensor:
+                n_rows: Optional[int] = None, out_name: str = "norm",
+                out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         R = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
-        out = ctx.buf(out_name, R, self.width, ctx.dtype)
+        out = ctx.buf(out_name, R, self.width, out_dtype or ctx.dtype)
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)
 
     def fusable_params(self):

@@ -185,7 +185,7 @@ def test_cancel_while_a_step_holds_a_reservation(models, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_named_intermediates_of_a_step(models, dtype):
     """The debug hook hands out (layer, stage, tensor) as the reference's does
-    (AbstractModel.java:122-128,1100-1107; TransformerBlock.java:177,189; CausalSelfAttention.java:299-301,384):
+    (AbstractModel.java:122-128,1100-1107; TransformerBlock.java:177,189; CausalSelfAttention.java:299-301,384,406):
     each against the plain model's value at that place."""
     m = models["B"]
     cfg, W = m.plain_cfg, m.W
@@ -209,12 +209,14 @@ def test_named_intermediates_of_a_step(models, dtype):
         scale = 1.0 / np.sqrt(D) / ((layer + 1) if cfg.get("scale_attn_by_inverse_layer_idx") else 1)
         att = P.causal_attention(qkv[:, :E], qkv[:, E:2 * E], qkv[:, 2 * E:], H, scale)
         assert np.abs(seen[(layer, "attention_value")] - att).max() < tol, layer
+        # the output projection before its bias (CausalSelfAttention.java:406)
+        assert np.abs(seen[(layer, "attention_output")] - att @ W[f"h.{layer}.attn.c_proj.weight"]).max() < tol, layer
         x1 = x + P.conv1d(att, W[f"h.{layer}.attn.c_proj.weight"], W[f"h.{layer}.attn.c_proj.bias"])
         assert np.abs(seen[(layer, "post_attention_residual")] - x1).max() < tol, layer
         x = P.block(x, W, layer, cfg)
         assert np.abs(seen[(layer, "post_ff_residual")] - x).max() < tol, layer
         assert np.abs(seen[(layer, "layer_output")] - x).max() < tol, layer
-    assert len(seen) == 1 + 7 * cfg["n_layer"]
+    assert len(seen) == 1 + 8 * cfg["n_layer"]
 
 
 @pytest.fixture(scope="module")

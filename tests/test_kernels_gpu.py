@@ -331,6 +331,29 @@ def test_attention_decode_with_keys_split_over_workgroups(ops, Hq, Hkv, D, page,
         ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, len(lens), Hq, scale, window, out, n_splits, ws[:10])
 
 
+@pytest.mark.parametrize("where", ["first", "share_end", helpers.quick("share_start"), "second_share_end", "last", "window_edge"])
+@pytest.mark.parametrize("D,page,window,n_splits", [helpers.quick(64, 16, None, 3), (144, 32, None, 2), (64, 16, 700, 4), (32, 64, 1500, 16)])
+def test_attention_decode_split_sees_one_far_key(ops, D, page, window, n_splits, where):
+    """One key among 2,100 carries nearly all the weight of the last query: a share's first or last key,
+    the sequence's first or last, or the oldest key that the window still holds.  Random keys alone give
+    near-uniform weights, under which a lost key moves the result by a thousandth."""
+    n = 2100
+    span = -(-(-(-n // page) * page) // n_splits // 64) * 64
+    far = {"first": 0, "share_end": span - 1, "share_start": span, "second_share_end": min(2 * span, n) - 1, "last": n - 1,
+           "window_edge": n - (window or n)}[where]
+    Hq, Hkv = 2, 1
+    case = PagedCase(lens=[n], new=[1], Hq=Hq, Hkv=Hkv, D=D, page=page, dtype=torch.bfloat16, seed=D + far, scale_boost=(far, 3.0))
+    scale = 0.7 / math.sqrt(D)
+    want = case.plain(scale, window)
+    seen = window is None or far >= n - window
+    if seen:      # the far key's value is the answer, nearly
+        assert np.abs(want[0, :D] - case.v[0][far].double().numpy()[:D]).max() < 0.1
+    out = torch.full_like(case.qcat, float("nan"))
+    ws = torch.full((ops.decode_workspace_floats(1, Hq, D, n_splits),), float("nan"), device=DEV)
+    ops.attention_decode(case.qcat, case.cache, case.bt, case.seq_lens, 1, Hq, scale, window, out, n_splits, ws)
+    assert np.abs(out.double().cpu().numpy() - want).max() < ATT_TOL[torch.bfloat16], (where, far)
+
+
 @pytest.mark.simt_quick
 def test_when_decode_attention_splits_its_keys(ops):
     assert ops.decode_splits(1, 12, 64, 16) == 1                   # 1,024 keys: one share

@@ -51,3 +51,34 @@ def test_random_configuration_mixed_and_whole(tmp_path, seed):
         s = helpers.trace_session(m.folder, dtype, -(-P // unit) * unit, page)
         got = helpers.replay(s, helpers.trace_whole(*reqs[-1]))
         helpers.check_against_plain(m, got, reqs[-1:], dtype, f"whole {cfg} page {page}")
+
+
+# (width, heads): head sizes 10, 24, 25 and 40; a width of 100 is no multiple of 8 either, so its products
+# leave the matrix cores as well
+@pytest.mark.parametrize("width,heads", [(40, 4), helpers.quick(72, 3), (100, 4), (120, 3)])
+def test_head_sizes_that_are_no_multiple_of_16(tmp_path, width, heads):
+    """config.json allows any n_embd / n_head: the 32-bit path takes every head size up to 256, and
+    bfloat16 serves those that the matrix-core attention kernels do not take through the plain
+    attention kernel (the reference divides likewise and asks nothing more of the head size:
+    safetensors/src/main/java/io/teknek/deliverance/safetensors/Config.java:340-354)."""
+    cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=width, n_head=heads,
+               vocab_size=211, n_positions=96, layer_norm_epsilon=1e-5, activation_function="gelu_new",
+               bos_token_id=0, eos_token_id=1)
+    m = helpers.make_model(tmp_path, cfg, seed=width)
+    reqs = [(f"r{i}", m.prompt(n, salt=i)) for i, n in enumerate((70, 9, 33, 95))]
+    steps = helpers.trace_mixed(reqs, seed=width, prefill_sizes=(9, 2, 40, 4), decode_tail=7)
+    for dtype in ("float32", "bfloat16"):
+        s = helpers.trace_session(m.folder, dtype, helpers.max_live_tokens(steps), poison_freed=True)
+        got = helpers.replay(s, steps)
+        helpers.check_against_plain(m, got, reqs, dtype, f"head size {width // heads}, mixed")
+        got = helpers.replay(s, helpers.trace_bulk_then_single(*reqs[3], 32))
+        helpers.check_against_plain(m, got, reqs[3:], dtype, f"head size {width // heads}, bulk+single")
+        s.cache.manager.check()
+
+
+def test_head_sizes_beyond_the_kernels_are_refused(tmp_path):
+    cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=1, n_embd=272, n_head=1,
+               vocab_size=50, n_positions=32)
+    m = helpers.make_model(tmp_path, cfg, seed=1)
+    with pytest.raises(ValueError, match="head size 272"):
+        helpers.trace_session(m.folder, "float32", 64)

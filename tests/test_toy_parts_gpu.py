@@ -39,7 +39,11 @@ def _register_once():
         return
 
     class RunningMean(Mixer):
-        """y_t = W . mean(h_0 .. h_t).  State per request: the sum so far (width floats) and the count."""
+        """y_t = W . mean(h_0 .. h_t).  State per request: the sum so far (width floats) and the count.
+        Everything it reads about the step lies on the device (the rows' sequences, the portions' first
+        rows, the sequences' state slots), so a decode step with this mixer is recorded and replayed
+        like any other."""
+        graph_safe = True
 
         def __init__(self, spec, params, dtype, device):
             self.width = spec.width
@@ -50,18 +54,18 @@ def _register_once():
 
         def forward(self, ctx, h, x, call):
             state = ctx.cache.state[call.cache]                       # [slots, width + 1], float32
-            means = ctx.buf("toy_means", h.shape[0], self.width, ctx.dtype)
-            for s in range(ctx.n_seqs):
-                a, b = ctx.q_start_host[s], ctx.q_start_host[s + 1]
-                slot = ctx.state_slots_host[s]
-                if slot < 0:
-                    continue                                          # a padding row of a fixed-shape step
-                run = torch.cumsum(h[a:b].float(), dim=0) + state[slot, :self.width]
-                count = state[slot, self.width] + torch.arange(1, b - a + 1, device=h.device, dtype=torch.float32)
-                means[a:b] = (run / count[:, None]).to(ctx.dtype)
-                if call.write:
-                    state[slot, :self.width] = run[-1]
-                    state[slot, self.width] = count[-1]
+            N, Wd = h.shape[0], self.width
+            before = ops.state_gather(state, ctx.state_slots, ctx.seq_of_token, ctx.buf("toy_before", N, Wd + 1, torch.float32))
+            first = ctx.q_start.long()[ctx.seq_of_token[:N].long()]   # the first row of each row's portion
+            c = torch.cumsum(h.float(), dim=0)
+            base = torch.where((first > 0)[:, None], c[(first - 1).clamp(min=0)], torch.zeros_like(c))
+            after = ctx.buf("toy_after", N, Wd + 1, torch.float32)
+            after[:, :Wd] = c - base + before[:, :Wd]
+            after[:, Wd] = before[:, Wd] + (torch.arange(N, device=h.device) - first + 1).float()
+            means = ctx.buf("toy_means", N, Wd, ctx.dtype)
+            means.copy_(after[:, :Wd] / after[:, Wd:])
+            if call.write:                                            # what a portion's last row leaves is the state
+                ops.state_scatter(state, ctx.state_slots, ctx.q_start, after, ctx.n_seqs)
             ops.linear(means, self.weight, None, x, accumulate=True)
 
     register_mixer("toy_running_mean", RunningMean)
@@ -178,6 +182,29 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_folder, dtype):
     a = helpers.replay(s, helpers.trace_whole("again", reqs[0][1]))["again"]
     b = helpers.replay(s, helpers.trace_whole("again", reqs[0][1]))["again"]
     assert np.array_equal(a, b)
+
+
+@pytest.mark.needs_device
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_decodes_from_recorded_graphs(toy_folder, dtype):
+    """The mixer with state inside recorded decode steps: batches of 5, 4, 3, 2, 1 padded to buckets and
+    replayed (every bucket several times, with eager prompt steps of later requests between the replays),
+    each step's logits against the plain model."""
+    from test_engine_paths_gpu import decode_trace
+    _, W = P.read_model_folder(toy_folder)
+    s = helpers.trace_session(toy_folder, dtype, 512, poison_freed=True, use_graphs=True, sample=True)
+    assert s.model.graph_safe and s.runner.use_graphs
+    rng = np.random.default_rng(4)
+    tol = {"float32": 2e-5, "bfloat16": 6e-2}[dtype]
+    for round_ in range(2):                     # the second round replays the graphs that the first recorded
+        reqs = [(f"g{round_}{i}", [int(t) for t in rng.integers(0, V, size=n)]) for i, n in enumerate((30, 17, 44, 9, 25))]
+        got = helpers.replay(s, decode_trace(reqs, [5, 9, 14, 3, 20]))
+        for rid, ids in reqs:
+            err = np.abs(got[rid] - plain_toy(W, ids)).max()
+            assert err < tol, f"round {round_} {rid}: {err}"
+        s.cache.manager.check()
+        assert s.cache.manager.live() == []
+    assert len(s.runner._graphs) >= 3
 
 
 @pytest.mark.needs_device
