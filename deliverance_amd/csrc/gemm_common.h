@@ -49,3 +49,9 @@ __device__ __forceinline__ void kv_scatter_store(const KvScatter& kv, int slot, 
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }
 
+
+// The tiles of 256 x 256 (gemm_wide.hip): what they take, where they pay, and their launch.
+bool da_gemm_wide_takes(int act, int accumulate, int out_dtype, int K);
+bool da_gemm_wide_pays(int M, int N);
+void da_gemm_wide_launch(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
+                         const KvScatter& kv, int M, int N, int K);

@@ -7,7 +7,7 @@
 //
 //  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
 //    buffers, with the next four slabs already in flight in registers.  For steps with many rows
-//    (prefill).
+//    (prefill).  Products that fill the chip with tiles of 256 x 256 go to gemm_wide.hip instead.
 //  * gemm_skinny: for M <= 64 (decode).  A workgroup owns 16 output columns; its wavefronts (4 to 12)
 //    split K, pull their part of a and w from memory in whole cache lines, pass it through LDS into
 //    MFMA 16x16x32 fragments and add their sums through LDS in a fixed order.  Bound by the bytes of w.
@@ -756,6 +756,12 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
     // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so
     // the choice does not change a result.
+    if (da_gemm_wide_takes(act, accumulate, out_dtype, K) && da_gemm_wide_pays(M, N)) {
+      // tiles of 256 x 256 where they fill the chip: the same sums in the same order, half the LDS traffic
+      da_gemm_wide_launch(s, A, lda, W, ldw, ep, kv, M, N, K);
+      DA_CHECK_LAUNCH("gemm_bf16");
+      return 0;
+    }
     const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
     const long tiles12864 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 64);
     // (up to 256 tiles a workgroup has its compute unit to itself: four slabs in flight instead of two, with the

@@ -163,6 +163,58 @@ def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
         assert (out - ref).abs().max() < tol, (act, acc, bias, od)
 
 
+@pytest.mark.parametrize("M,N,K", [helpers.quick(300, 200, 128), (257, 520, 64), (2048, 1600, 320), (700, 4800, 192)])
+def test_gemm_wide_tiles(ops, M, N, K):
+    """The tiles of 256 x 256 (operands from memory straight into LDS, two stages): every epilogue against
+    64-bit arithmetic, and bit for bit what the 128 x 128 tiles give (both sum over k in ascending steps
+    of 16); edges in M and N, one slab, odd and even numbers of slabs."""
+    g = torch.Generator().manual_seed(M + N + K)
+    wide = lambda *a_, **k_: ops.linear_mfma(*a_, form="wide", **k_)
+    for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
+                               ("gelu", False, False, torch.bfloat16), (None, True, True, torch.float32),
+                               (None, False, False, torch.float32), ("silu", False, True, torch.bfloat16)):
+        out, ref = _gemm_case(ops, wide, M, N, K, torch.bfloat16, act, acc, bias, od, g)
+        tol = (1e-2 if od == torch.bfloat16 else 1e-4) * max(1.0, ref.abs().max().item())
+        assert (out - ref).abs().max() < tol, (act, acc, bias, od)
+    a = bf(torch.randn(M, K, generator=g) * 0.5).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.2).to(DEV)
+    b = bf(torch.randn(N, generator=g)).to(DEV)
+    for od, acc in ((torch.bfloat16, False), (torch.float32, True)):
+        o1 = torch.full((M, N), 0.25, device=DEV, dtype=od)
+        o2 = o1.clone()
+        ops.linear_mfma(a, w, b, o1, None, acc, form="wide")
+        ops.linear_mfma(a, w, b, o2, None, acc)
+        assert torch.equal(o1, o2), (od, acc)
+    with pytest.raises(ops.KernelError, match="multiple of 64"):
+        ops.linear_mfma(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous(), b, o1, form="wide")
+
+
+@pytest.mark.parametrize("M", [helpers.quick(300), 1000])
+def test_gemm_wide_tiles_write_keys_and_values(ops, M):
+    g = torch.Generator().manual_seed(M)
+    Hq, Hkv, D, page, K = 5, 3, 48, 16, 128
+    N = (Hq + 2 * Hkv) * D
+    n_pages = (M + page - 1) // page + 2
+    a = bf(torch.randn(M, K, generator=g)).to(DEV)
+    w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
+    bias = bf(torch.randn(N, generator=g)).to(DEV)
+    perm = torch.randperm(n_pages * page, generator=g)[:M].to(torch.int32)
+    perm[M // 2] = -1
+    runs = torch.cat([torch.arange(16, 16 + M // 2), torch.arange(16 + M // 2 + 19, 16 + M // 2 + 19 + M - M // 2)]).to(torch.int32)
+    runs[M // 4] = -1
+    for order in (perm, runs):
+        slots = order.to(DEV)
+        c1 = torch.zeros(n_pages + 2, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
+        c2 = torch.zeros_like(c1)
+        out1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+        out2 = torch.empty_like(out1)
+        ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D, form="wide")
+        ops.linear_mfma(a, w, bias, out2)
+        ops.kv_write(out2, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)
+        assert torch.equal(out1, out2)
+        assert torch.equal(c1, c2) and c1.abs().sum() > 0
+
+
 @pytest.mark.simt_quick
 @pytest.mark.parametrize("M", [20, 200])
 def test_gemm_into_rows_longer_than_the_result(ops, M):
