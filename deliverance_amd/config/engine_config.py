@@ -42,6 +42,7 @@ class EngineConfig:
     state_slots: Optional[int] = None  # slots for fixed-size per-request state; None: max_num_seqs
     use_graphs: bool = True            # replay decode-only steps from captured HIP graphs
     run_ahead: bool = True             # launch the next decode step before the running one's tokens are read
+    native_step: bool = True           # the layer loop in one call into the library where the parts allow it
     poison_freed_pages: bool = False   # debug: a page that goes back is filled with NaN again
     device: str = "cuda:0"
 

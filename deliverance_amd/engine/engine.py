@@ -77,7 +77,8 @@ class CausalLanguageModel:
         self.cache = DeviceCache(needs, model.dtype, model.device, engine_config.page_size, tokens, n_slots,
                                  poison_freed=engine_config.poison_freed_pages)
         self.runner = StepRunner(model, self.cache, use_graphs=engine_config.use_graphs,
-                                 max_graph_batch=max(engine_config.max_num_seqs, 1), kernels=engine_config.kernels)
+                                 max_graph_batch=max(engine_config.max_num_seqs, 1), kernels=engine_config.kernels,
+                                 native_step=engine_config.native_step)
         self.scheduler = Scheduler(self.cache.manager, model.config.max_positions, model.config.eos_token_ids,
                                    engine_config.max_num_seqs, engine_config.max_batch_tokens,
                                    engine_config.max_chunk, on_open=self.cache.reset_state)

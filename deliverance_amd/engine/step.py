@@ -153,10 +153,16 @@ class StepPacker:
 
 class StepRunner:
     def __init__(self, model: CausalLM, cache: DeviceCache, use_graphs: bool = False, max_graph_batch: int = 256,
-                 kernels: str = "tuned"):
+                 kernels: str = "tuned", native_step: bool = True):
         self.model = model
         self.cache = cache
         self.kernels = kernels                       # "tuned" | "reference" (EngineConfig.kernels)
+        # the layer loop in one call into the library, where the model's parts allow it (engine/native_step.py)
+        self.native = None
+        if native_step:
+            from .native_step import NativeStep
+            if NativeStep.takes(model, cache, kernels):
+                self.native = NativeStep(model, cache)
         # hook(layer, stage, tensor) for named intermediates of every step; steps then run kernel by
         # kernel, never from a recorded graph
         self.debug_hook = None
@@ -295,8 +301,16 @@ class StepRunner:
         R = meta["R"]
         if any(e.from_sampled is not None for e in entries):
             ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, self.model.config.vocab_size)
-        logits = self.model.forward(ctx, ctx.want_rows if R else None, R)
+        logits = self._forward(ctx, ctx.want_rows if R else None, R)
         return logits, ctx
+
+    def _forward(self, ctx, want_rows, n_want):
+        """The model's forward pass of this step: from C++ in one call, or part by part (always with the
+        debug hook or the kernel profiler, which look between the kernels)."""
+        from ..profiler import KernelProfiler
+        if self.native is not None and ctx.debug_hook is None and not KernelProfiler.enabled:
+            return self.native.forward(ctx, want_rows, n_want)
+        return self.model.forward(ctx, want_rows, n_want)
 
     def _context(self, dev, offs, meta, arena) -> StepContext:
         def view(name):
@@ -355,7 +369,7 @@ class StepRunner:
 
         def body():
             ops.take_tokens(ctx.tokens, ctx.token_src, self.sampled, self.model.config.vocab_size)
-            logits = self.model.forward(ctx, ctx.want_rows, bucket)
+            logits = self._forward(ctx, ctx.want_rows, bucket)
             ops.sample(logits, ctx.extra, sampled)
             return logits
 

@@ -85,6 +85,9 @@ _ARGTYPES = {
     "da_attn_decode_split": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
     "da_attn_prefill": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP],
     "da_sample": [_VP, _I, _I, _I, _VP, _VP, _VP],
+    "da_decode_splits": [_I, _I, _I, _I],
+    "da_can_fuse_ln": [_I, _I, _I],
+    "da_run_step": [_VP, _VP],
     "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
 }
 _LIB = None
@@ -450,23 +453,16 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     return out
 
 
-# Measured on MI355X inside the model: the fused kernel wins up to 16 rows (one row tile) and a
-# width of 1024, by 10 to 15 % of a decode step; up to 8 rows (which take half the LDS, so that the
-# workgroups still run side by side) up to a width of 1280, and a single row up to 2048; beyond, the
-# separate norm and product are faster (every 16 output columns read and normalise all rows again:
-# at a width of 1600 and 8 rows 8.0 us against 3.1 + 3.9).
-FUSED_LN_LIMITS = ((16, 1024), (8, 1280), (1, 2048))       # (rows, width): fused up to these
-FUSED_LN_MAX_N = 16384      # ... and never for a vocabulary
+# Which steps the fused norm + product kernel takes (few rows, a width it holds; measured limits) is the
+# library's rule, da_can_fuse_ln in csrc/run_step.hip, so that the parts here and the step issued from C++
+# decide alike.
 FUSED_LN_KERNEL_MAX_ROWS = 32
 
 
 def can_fuse_ln(n_rows: int, x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether ``linear_ln`` takes this step: few rows, bfloat16 weights, a width the kernel holds."""
-    K = w.shape[1]
-    fits = any(n_rows <= r and K <= k for r, k in FUSED_LN_LIMITS)
-    return (_MODE == "tuned" and w.dtype == torch.bfloat16 and 0 < n_rows and fits
-            and K % 8 == 0 and w.shape[0] <= FUSED_LN_MAX_N
-            and w.stride(0) % 8 == 0 and x.dtype == torch.float32)
+    return (_MODE == "tuned" and w.dtype == torch.bfloat16 and x.dtype == torch.float32 and w.stride(0) % 8 == 0
+            and bool(_lib().da_can_fuse_ln(int(n_rows), int(w.shape[1]), int(w.shape[0]))))
 
 
 def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_weight: torch.Tensor,
@@ -544,20 +540,11 @@ def _attn_common(q, cache_slot, block_table, n_heads, out, name):
     return Hkv, page, D
 
 
-# Decode attention splits a (sequence, head) pair's keys over workgroups when the pairs alone leave most
-# of the chip idle and the context is long: shares of at least DECODE_SPLIT_MIN_KEYS keys, as many as
-# bring the workgroups to about DECODE_SPLIT_WORKGROUPS.  The choice reads the step's shape only (pairs
-# and the width of the block table), so that a recorded step keeps it.
-DECODE_SPLIT_MIN_KEYS = 1024
-DECODE_SPLIT_WORKGROUPS = 512
-DECODE_SPLIT_MAX = 32
-
-
 def decode_splits(n_seqs: int, n_heads: int, max_blocks: int, page: int) -> int:
-    by_keys = (max_blocks * page) // DECODE_SPLIT_MIN_KEYS
-    by_fill = DECODE_SPLIT_WORKGROUPS // max(1, n_seqs * n_heads)
-    n = min(by_keys, by_fill, DECODE_SPLIT_MAX)
-    return n if n >= 2 else 1
+    """How many workgroups share a (sequence, head) pair's keys in decode attention (1: one workgroup a
+    pair).  The library's rule (da_decode_splits in csrc/run_step.hip): from the step's shape only (pairs
+    and the width of the block table), so that a recorded step keeps it."""
+    return int(_lib().da_decode_splits(int(n_seqs), int(n_heads), int(max_blocks), int(page)))
 
 
 def attention_decode(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor,

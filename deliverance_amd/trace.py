@@ -30,7 +30,8 @@ class TraceSession:
     graph; ``last_sampled`` then holds the tokens that the device picked."""
 
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
-                 poison_freed: bool = False, kernels: str = "tuned", use_graphs: bool = False, sample: bool = False):
+                 poison_freed: bool = False, kernels: str = "tuned", use_graphs: bool = False, sample: bool = False,
+                 native_step: bool = True):
         import torch
         from . import models  # noqa: F401  (registers the architectures)
         from .config.engine_config import KERNEL_MODES
@@ -44,13 +45,14 @@ class TraceSession:
         # hold every live request whatever its length.
         self.cache = DeviceCache(self.model.cache_needs(), tdtype, device, page_size, max(max_tokens, 64),
                                  n_state_slots=8, poison_freed=poison_freed)
+        self.native_step = native_step
         self.runner = self._make_runner(use_graphs, kernels)
         self.sample = sample or use_graphs
         self.last_sampled = None
 
     def _make_runner(self, use_graphs: bool, kernels: str):
         from .engine.step import StepRunner
-        return StepRunner(self.model, self.cache, use_graphs=use_graphs, kernels=kernels)
+        return StepRunner(self.model, self.cache, use_graphs=use_graphs, kernels=kernels, native_step=self.native_step)
 
     def _drain(self):
         import torch
