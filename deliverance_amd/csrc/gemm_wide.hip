@@ -25,12 +25,8 @@
 #include <da_lds_dma.h>
 #include <type_traits>
 
-#define WD_BM 256
-#define WD_BN 256
 #define WD_BK 64
 #define WD_ROW_BYTES (WD_BK * 2)
-#define WD_HALF_BYTES (256 * WD_ROW_BYTES)       // a slab of a, or of w, in LDS: 32 KB
-#define WD_THREADS 512
 #define WD_REGION_BYTES 8960          // a wavefront's piece of LDS in the epilogue: 32 x 68 floats, then 32 places
 
 __device__ __forceinline__ void wave_lds_sync() {
@@ -40,9 +36,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 // OUTMODE: 0 bf16 store, 1 f32 store, 2 f32 +=
-template <int TN, int ACT, int OUTMODE>
+template <int TM, int TN, int ACT, int OUTMODE>
 __device__ __forceinline__ void
-wide_epilogue(floatx16 (&acc)[4][TN], const float (&bias)[TN], char* region, const void* safe, const Epilogue& ep,
+wide_epilogue(floatx16 (&acc)[TM][TN], const float (&bias)[TN], char* region, const void* safe, const Epilogue& ep,
               const KvScatter& kv, int M, int N, int mw, int nw, int lane) {
   constexpr int WC = 32 * TN;                                   // the wavefront's columns
   constexpr int ES = OUTMODE == 0 ? 2 : 4, CH = 16 / ES;       // bytes an element; elements a 16-byte piece
@@ -169,25 +165,34 @@ wide_epilogue(floatx16 (&acc)[4][TN], const float (&bias)[TN], char* region, con
     wave_lds_sync();       // the next pass parks over what this one read
   };
   pass(std::integral_constant<int, 0>{});
-  pass(std::integral_constant<int, 1>{});
-  pass(std::integral_constant<int, 2>{});
-  pass(std::integral_constant<int, 3>{});
+  if (TM > 1) pass(std::integral_constant<int, (TM > 1 ? 1 : 0)>{});
+  if (TM > 2) pass(std::integral_constant<int, (TM > 2 ? 2 : 0)>{});
+  if (TM > 3) pass(std::integral_constant<int, (TM > 3 ? 3 : 0)>{});
 }
 
-// Eight wavefronts: 2 in m x 4 in n, each 128 x 64.  (Four of 128 x 128 read a third less from LDS and
-// measured 15 to 25 % slower: one wavefront a SIMD has nobody to fill its waits.)
-template <int ACT, int OUTMODE>
-__global__ void __launch_bounds__(WD_THREADS)
+// BM x BN: the tile; WM x WN wavefronts of (BM / WM) x (BN / WN) each.  In use: 256 x 256 with 2 x 4
+// wavefronts of 128 x 64, one workgroup a compute unit (160 KB of LDS).  Measured beside it: four wavefronts
+// of 128 x 128 (a third less LDS traffic; 15 to 25 % slower: one wavefront a SIMD has nobody to fill its
+// waits); tiles of 128 x 128 with 2 x 2 wavefronts of 64 x 64, two workgroups a compute unit (80 KB each):
+// 5 to 15 % ahead of gemm_mfma.hip's tiles when timed alone from 200 tiles on, level or behind inside the
+// model, where a and w both come from memory: a slab of such a tile is half a microsecond of products,
+// and one or two slabs ahead do not cover the way from memory (gemm_mfma.hip keeps four in registers).
+template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
+__global__ void __launch_bounds__(WM * WN * 64)
 gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                  Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
-  // Two stages of a slab of a, three of a slab of w (32 KB each: all 160 KB of a compute unit).  The rows
-  // of a were written by the kernel before and come from a cache; w comes from memory for the first
-  // time and needs the longer way ahead.
-  __shared__ __attribute__((aligned(1024))) char smem[5 * WD_HALF_BYTES];
-  constexpr int NW = 8, TN = 2;
-  static_assert(NW * WD_REGION_BYTES <= 5 * WD_HALF_BYTES, "the epilogue regions fit the stages");
+  // Two stages of a slab of a, three of a slab of w.  The rows of a were written by the kernel before and
+  // come from a cache; w comes from memory for the first time and needs the longer way ahead.
+  constexpr int A_BYTES = BM * WD_ROW_BYTES, W_BYTES = BN * WD_ROW_BYTES;      // a slab of a, of w, in LDS
+  constexpr int NW = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int CA = BM / 8 / NW, CW = BN / 8 / NW;                             // copies a wavefront and slab
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && NW % 2 == 0,
+                "the tile does not split over the wavefronts");
+  static_assert(BN / WN == 64, "the epilogue parks 64 columns a wavefront");
+  __shared__ __attribute__((aligned(1024))) char smem[2 * A_BYTES + 3 * W_BYTES];
+  static_assert(NW * WD_REGION_BYTES <= 2 * A_BYTES + 3 * W_BYTES, "the epilogue regions fit the stages");
   char* const smem_a = smem;
-  char* const smem_w = smem + 2 * WD_HALF_BYTES;
+  char* const smem_w = smem + 2 * A_BYTES;
 
   // Each XCD (workgroups that follow each other in launch order land on different ones) takes a
   // contiguous run of tiles, m fastest, so that its workgroups share slabs of w in its L2.
@@ -198,59 +203,59 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
     const int xcd = pid % 8, local = pid / 8;
     pid = xcd * per + (xcd < rem ? xcd : rem) + local;
   }
-  const int m0 = (pid % tiles_m) * WD_BM, n0 = (pid / tiles_m) * WD_BN;
+  const int m0 = (pid % tiles_m) * BM, n0 = (pid / tiles_m) * BN;
 
   const int t = threadIdx.x, lane = t % 64;
   const int wave = __builtin_amdgcn_readfirstlane(t / 64);
-  const int wm = (wave % 2) * 128, wn = (wave / 2) * 64;
+  const int wm = (wave % WM) * (BM / WM), wn = (wave / WM) * (BN / WN);
   const int fr = lane % 32, fk = lane / 32;
 
-  // Copies: a stage of a (of w) is 32 blocks of 8 rows; wavefront v takes blocks v, v + 8, v + 16, v + 24.
+  // Copies: a stage of a (of w) is BM / 8 (BN / 8) blocks of 8 rows; wavefront v takes blocks v, v + NW, ...
   // Lane l of a copy stands for row l / 8 of the block and position l % 8 of that row, which holds the
   // row's piece (l % 8) ^ (r / 2 % 8), r the row's number in the stage.  Rows past the edge of a or w read
   // the last row: what they give is never stored.
-  const bf16_t* src_a[4];
-  const bf16_t* src_w[4];
-  int blk[4];                                        // byte offset of the wavefront's blocks in a stage
+  const bf16_t* src_a[CA];
+  const bf16_t* src_w[CW];
+  int blk[CA > CW ? CA : CW];                        // byte offset of the wavefront's blocks in a stage
   {
-    // (row r of a stage is row l / 8 of block v + 8 i: r / 2 % 8 = (4 (v % 2) + l / 16) % 8)
+    // (row r of a stage is row l / 8 of block v + NW i, NW even: r / 2 % 8 = (4 (v % 2) + l / 16) % 8)
     const int rl = lane / 8, piece = (lane % 8) ^ ((4 * (wave & 1) + (rl >> 1)) & 7);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < (CA > CW ? CA : CW); ++i) {
       const int b = i * NW + wave;
       const int ra = m0 + b * 8 + rl, rw = n0 + b * 8 + rl;
-      src_a[i] = a + (size_t)(ra < M ? ra : M - 1) * lda + piece * 8;
-      src_w[i] = w + (size_t)(rw < N ? rw : N - 1) * ldw + piece * 8;
+      if (i < CA) src_a[i] = a + (size_t)(ra < M ? ra : M - 1) * lda + piece * 8;
+      if (i < CW) src_w[i] = w + (size_t)(rw < N ? rw : N - 1) * ldw + piece * 8;
       blk[i] = b * 1024;
     }
   }
-#define WD_COPY_A(i, stage) { lds_dma16(src_a[i], smem_a + (stage) * WD_HALF_BYTES + blk[i]); src_a[i] += WD_BK; }
-#define WD_COPY_W(i, stage) { lds_dma16(src_w[i], smem_w + (stage) * WD_HALF_BYTES + blk[i]); src_w[i] += WD_BK; }
+#define WD_COPY_A(i, stage) { lds_dma16(src_a[i], smem_a + (stage) * A_BYTES + blk[i]); src_a[i] += WD_BK; }
+#define WD_COPY_W(i, stage) { lds_dma16(src_w[i], smem_w + (stage) * W_BYTES + blk[i]); src_w[i] += WD_BK; }
 
   // Fragments: lane l gives row l % 32 of a 32-row piece and the 8 k from 8 * (l / 32) of a k-step:
   // piece 2 * step + l / 32 of its row, stored at that number ^ (row / 2 % 8).
-  int a_off[4], w_off[TN], k_off[4];
+  int a_off[TM], w_off[TN], k_off[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) a_off[i] = (wm + i * 32 + fr) * WD_ROW_BYTES;
+  for (int i = 0; i < TM; ++i) a_off[i] = (wm + i * 32 + fr) * WD_ROW_BYTES;
 #pragma unroll
   for (int j = 0; j < TN; ++j) w_off[j] = (wn + j * 32 + fr) * WD_ROW_BYTES;
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) k_off[ks] = ((2 * ks + fk) ^ ((fr >> 1) & 7)) * 16;
 #define WD_READ(FA, FB, sa, sw, ks)                                                                                  \
   {                                                                                                                  \
-    const char* pa = smem_a + (sa) * WD_HALF_BYTES + k_off[ks];                                                      \
-    const char* pw = smem_w + (sw) * WD_HALF_BYTES + k_off[ks];                                                      \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) FA[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(pa + a_off[i])); \
+    const char* pa = smem_a + (sa) * A_BYTES + k_off[ks];                                                            \
+    const char* pw = smem_w + (sw) * W_BYTES + k_off[ks];                                                            \
+    _Pragma("unroll") for (int i = 0; i < TM; ++i) FA[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(pa + a_off[i])); \
     _Pragma("unroll") for (int j = 0; j < TN; ++j) FB[j] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(pw + w_off[j])); \
   }
 #define WD_MFMA1(FA, FB, q) \
   acc[(q) / TN][(q) % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[(q) / TN], FB[(q) % TN], acc[(q) / TN][(q) % TN], 0, 0, 0)
-#define WD_MFMA(FA, FB) { _Pragma("unroll") for (int q = 0; q < 4 * TN; ++q) WD_MFMA1(FA, FB, q); }
+#define WD_MFMA(FA, FB) { _Pragma("unroll") for (int q = 0; q < TM * TN; ++q) WD_MFMA1(FA, FB, q); }
 #define WD_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-  floatx16 acc[4][TN];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -277,22 +282,23 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
   // and w(s + 3) into the stages that slab s left.  Copies land in the order they were asked for, so
   // "slab s + 1 is there" is "at most the four youngest copies, w(s + 2), are still under way".
   const int nslab = K / WD_BK;
-  bf16x8_t fa0[4], fb0[TN], fa1[4], fb1[TN];
+  bf16x8_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) WD_COPY_A(i, 0);
+  for (int i = 0; i < CA; ++i) WD_COPY_A(i, 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) WD_COPY_W(i, 0);
+  for (int i = 0; i < CW; ++i) WD_COPY_W(i, 0);
   if (nslab > 1) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) WD_COPY_A(i, 1);
+    for (int i = 0; i < CA; ++i) WD_COPY_A(i, 1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) WD_COPY_W(i, 1);
+    for (int i = 0; i < CW; ++i) WD_COPY_W(i, 1);
   }
   if (nslab > 2) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) WD_COPY_W(i, 2);
+    for (int i = 0; i < CW; ++i) WD_COPY_W(i, 2);
   }
-  if (nslab > 2) DA_WAIT_VMCNT(12); else if (nslab > 1) DA_WAIT_VMCNT(8); else DA_WAIT_VMCNT(0);
+  static_assert(CA + 2 * CW <= 15, "the count of copies under way fits its field");
+  if (nslab > 2) DA_WAIT_VMCNT(CA + 2 * CW); else if (nslab > 1) DA_WAIT_VMCNT(CA + CW); else DA_WAIT_VMCNT(0);
   __builtin_amdgcn_s_barrier();
   WD_READ(fa0, fb0, 0, 0, 0);
   int sw = 0;                                          // the stage of w that holds slab s
@@ -308,7 +314,7 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
     WD_READ(fa1, fb1, sa, sw, 1);
     WD_FENCE();
 #pragma unroll
-    for (int q = 1; q < 4 * TN; ++q) WD_MFMA1(fa0, fb0, q);
+    for (int q = 1; q < TM * TN; ++q) WD_MFMA1(fa0, fb0, q);
     WD_FENCE();
     WD_READ(fa0, fb0, sa, sw, 2);
     WD_FENCE();
@@ -320,18 +326,23 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
     WD_FENCE();
     // Slab s + 1 must have landed, and every wavefront must be done reading slab s, before a(s + 2) and
     // w(s + 3) take its place: one barrier for both.
-    if (COPY_A) DA_WAIT_VMCNT(4); else DA_WAIT_VMCNT(0);      // (COPY_A: the tail before this one asked for w(s + 2) last)
+    if (COPY_A) DA_WAIT_VMCNT(CW); else DA_WAIT_VMCNT(0);     // (COPY_A: the tail before this one asked for w(s + 2) last)
     __builtin_amdgcn_s_waitcnt(0xC07F);                        // lgkmcnt(0): this wavefront's reads of slab s are complete
     __builtin_amdgcn_s_barrier();
     // The slab's last k-step, its products one by one, and between them the copies and the reads of slab
     // s + 1's first fragments: the matrix cores have work while the wavefront issues the rest.
+    constexpr int CPQ = (CA + CW + TM * TN - 1) / (TM * TN);      // copies after each product
+    static_assert(TM + TN <= TM * TN, "a read for every product at most");
 #pragma unroll
-    for (int q = 0; q < 4 * TN; ++q) {
+    for (int q = 0; q < TM * TN; ++q) {
       WD_MFMA1(fa1, fb1, q);
-      if (COPY_A && q < 4) WD_COPY_A(q, sa);
-      if (COPY_W && q >= 4) WD_COPY_W(q - 4, sw);
-      if (NEXT && q < 4) fa0[q] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_a + (sa ^ 1) * WD_HALF_BYTES + k_off[0] + a_off[q]));
-      if (NEXT && q >= 4 && q < 4 + TN) fb0[q - 4] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_w + sw1 * WD_HALF_BYTES + k_off[0] + w_off[q - 4]));
+#pragma unroll
+      for (int c = q * CPQ; c < (q + 1) * CPQ; ++c) {             // (all of a's before all of w's)
+        if (COPY_A && c < CA) WD_COPY_A(c, sa);
+        if (COPY_W && c >= CA && c < CA + CW) WD_COPY_W(c - CA, sw);
+      }
+      if (NEXT && q < TM) fa0[q] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_a + (sa ^ 1) * A_BYTES + k_off[0] + a_off[q]));
+      if (NEXT && q >= TM && q < TM + TN) fb0[q - TM] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_w + sw1 * W_BYTES + k_off[0] + w_off[q - TM]));
       WD_FENCE();
     }
     sw = sw1;
@@ -352,20 +363,32 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
 #undef WD_MFMA1
 #undef WD_FENCE
   // (the last barrier of the loop: nobody reads the stages any more)
-  wide_epilogue<TN, ACT, OUTMODE>(acc, bias, smem + wave * WD_REGION_BYTES, (const void*)w, ep, kv, M, N, m0 + wm, n0 + wn, lane);
+  wide_epilogue<TM, TN, ACT, OUTMODE>(acc, bias, smem + wave * WD_REGION_BYTES, (const void*)w, ep, kv, M, N, m0 + wm, n0 + wn, lane);
 }
 
-template <int ACT>
+template <int BM, int BN, int WM, int WN, int ACT>
 static void launch_wide_act(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
                             const KvScatter& kv, int M, int N, int K) {
-  const int tiles_m = da_ceil_div(M, WD_BM), tiles_n = da_ceil_div(N, WD_BN);
-  const dim3 grid(tiles_m * tiles_n), block(WD_THREADS);
+  const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
+  const dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if (ep.accumulate)
-    hipLaunchKernelGGL((gemm_wide_kernel<DA_ACT_NONE, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_wide_kernel<BM, BN, WM, WN, DA_ACT_NONE, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else if (ep.out_dtype == DA_F32)
-    hipLaunchKernelGGL((gemm_wide_kernel<DA_ACT_NONE, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_wide_kernel<BM, BN, WM, WN, DA_ACT_NONE, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
   else
-    hipLaunchKernelGGL((gemm_wide_kernel<ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_wide_kernel<BM, BN, WM, WN, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+}
+
+template <int BM, int BN, int WM, int WN>
+static void launch_wide(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
+                        const KvScatter& kv, int M, int N, int K) {
+  switch (ep.act) {
+    case DA_ACT_GELU_TANH: launch_wide_act<BM, BN, WM, WN, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_GELU_ERF: launch_wide_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_RELU: launch_wide_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_SILU: launch_wide_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    default: launch_wide_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+  }
 }
 
 // What the wide tiles take: K in whole slabs, and an activation only with a bfloat16 result (the forms
@@ -379,20 +402,14 @@ bool da_gemm_wide_takes(int act, int accumulate, int out_dtype, int K) {
 // from 152 tiles on (N = 4,800: 39 against 47 us; N = 6,400, 200 tiles: 42 against 62 us), behind at 128
 // tiles and fewer (N = 4,096: 30 against 27 us).
 bool da_gemm_wide_pays(int M, int N) {
-  const long tiles = (long)da_ceil_div(M, WD_BM) * da_ceil_div(N, WD_BN);
+  const long tiles = (long)da_ceil_div(M, 256) * da_ceil_div(N, 256);
   const long rounds = (tiles + 255) / 256;
   return tiles * 100 >= rounds * 256 * 55;
 }
 
 void da_gemm_wide_launch(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
                          const KvScatter& kv, int M, int N, int K) {
-  switch (ep.act) {
-    case DA_ACT_GELU_TANH: launch_wide_act<DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_GELU_ERF: launch_wide_act<DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_RELU: launch_wide_act<DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_SILU: launch_wide_act<DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    default: launch_wide_act<DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-  }
+  launch_wide<256, 256, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
 }
 
 // The wide tiles alone, whatever the shape (tests and timing call it; da_gemm_bf16 chooses by shape).

@@ -422,8 +422,8 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
                 slot_map: Optional[torch.Tensor] = None, q_cols: int = 0, form: str = "auto") -> torch.Tensor:
     """out (+)= act(a @ w.T + bias) on the matrix cores; a, w bfloat16, K a multiple of 8.  With
     ``kv_cache`` the columns from ``q_cols`` on (k | v) also go to the cache rows ``slot_map``.
-    ``form``: "auto" lets the library choose by shape; "wide" asks for the tiles of 256 x 256 whatever
-    the shape (K a multiple of 64; tests and timing)."""
+    ``form``: "auto" lets the library choose by shape; "wide" asks for the tiles of 256 x 256 whose
+    operands go from memory straight into LDS, whatever the shape (K a multiple of 64; tests and timing)."""
     _dev(a, w, bias, out)
     _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
     M, K = a.shape

@@ -164,12 +164,12 @@ def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [helpers.quick(300, 200, 128), (257, 520, 64), (2048, 1600, 320), (700, 4800, 192)])
-def test_gemm_wide_tiles(ops, M, N, K):
-    """The tiles of 256 x 256 (operands from memory straight into LDS, two stages): every epilogue against
-    64-bit arithmetic, and bit for bit what the 128 x 128 tiles give (both sum over k in ascending steps
-    of 16); edges in M and N, one slab, odd and even numbers of slabs."""
+def test_gemm_wide_tiles(ops, M, N, K, form="wide"):
+    """The tiles of 256 x 256 whose operands go from memory straight into LDS (two stages of a, three of
+    w): every epilogue against 64-bit arithmetic, and bit for bit what the other tile forms give (all sum
+    over k in ascending steps of 16); edges in M and N, one to five slabs."""
     g = torch.Generator().manual_seed(M + N + K)
-    wide = lambda *a_, **k_: ops.linear_mfma(*a_, form="wide", **k_)
+    wide = lambda *a_, **k_: ops.linear_mfma(*a_, form=form, **k_)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
                                ("gelu", False, False, torch.bfloat16), (None, True, True, torch.float32),
                                (None, False, False, torch.float32), ("silu", False, True, torch.bfloat16)):
@@ -182,15 +182,15 @@ def test_gemm_wide_tiles(ops, M, N, K):
     for od, acc in ((torch.bfloat16, False), (torch.float32, True)):
         o1 = torch.full((M, N), 0.25, device=DEV, dtype=od)
         o2 = o1.clone()
-        ops.linear_mfma(a, w, b, o1, None, acc, form="wide")
+        ops.linear_mfma(a, w, b, o1, None, acc, form=form)
         ops.linear_mfma(a, w, b, o2, None, acc)
         assert torch.equal(o1, o2), (od, acc)
     with pytest.raises(ops.KernelError, match="multiple of 64"):
-        ops.linear_mfma(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous(), b, o1, form="wide")
+        ops.linear_mfma(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous(), b, o1, form=form)
 
 
 @pytest.mark.parametrize("M", [helpers.quick(300), 1000])
-def test_gemm_wide_tiles_write_keys_and_values(ops, M):
+def test_gemm_wide_tiles_write_keys_and_values(ops, M, form="wide"):
     g = torch.Generator().manual_seed(M)
     Hq, Hkv, D, page, K = 5, 3, 48, 16, 128
     N = (Hq + 2 * Hkv) * D
@@ -208,7 +208,7 @@ def test_gemm_wide_tiles_write_keys_and_values(ops, M):
         c2 = torch.zeros_like(c1)
         out1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
         out2 = torch.empty_like(out1)
-        ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D, form="wide")
+        ops.linear_mfma(a, w, bias, out1, kv_cache=c1, slot_map=slots, q_cols=Hq * D, form=form)
         ops.linear_mfma(a, w, bias, out2)
         ops.kv_write(out2, Hq * D, (Hq + Hkv) * D, c2, slots, Hkv, D)
         assert torch.equal(out1, out2)
