@@ -105,8 +105,8 @@ def engine_from_gpu_weights(cfg, dtype, seats, seed=0, **kw):
     del tensors
     kw.setdefault("max_batch_tokens", max(2048, seats))
     kw.setdefault("max_chunk", 1024)
-    ec = EngineConfig(dtype=dtype, max_num_seqs=max(seats, 2), max_cached_tokens=max(seats, 2) * cfg["n_positions"],
-                      page_size=16, **kw)
+    pool = kw.pop("max_cached_tokens", max(seats, 2) * cfg["n_positions"])
+    ec = EngineConfig(dtype=dtype, max_num_seqs=max(seats, 2), max_cached_tokens=pool, page_size=16, **kw)
     return CausalLanguageModel(model, ec)
 
 
@@ -144,14 +144,15 @@ def decode_run(model, cfg, rng, batch, prompt_len, steps, warmup):
     return dt, ctx_mean
 
 
-def prefill_run(model, cfg, rng, dkey):
-    """2 x 1,024-token prompts in ONE step of the engine's step function, logits at the two last rows."""
+def prefill_run(model, cfg, rng, dkey, n_prompts=2, length=1024):
+    """``n_prompts`` x ``length``-token prompts (2 x 1,024 unless asked otherwise) in ONE step of the engine's step
+    function, logits at the last row of each."""
     import torch
     from deliverance_amd.engine.step import StepEntry
     times = []
     for it in range(5):                       # the first rounds warm up; the best of the rest counts
-        entries = [StepEntry(f"prefill{i}", [int(t) for t in rng.integers(0, cfg["vocab_size"], size=1024)], [1023])
-                   for i in range(2)]
+        entries = [StepEntry(f"prefill{i}", [int(t) for t in rng.integers(0, cfg["vocab_size"], size=length)], [length - 1])
+                   for i in range(n_prompts)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         model.runner.run(entries)
@@ -160,8 +161,9 @@ def prefill_run(model, cfg, rng, dkey):
         for e in entries:
             model.cache.manager.close(e.rid)
     t = min(times[2:])
-    fl = step_flops(cfg, [1024, 1024])
-    return {"value": round(2048 / t, 1), "tokens": 2048, "ms": round(t * 1e3, 3), "frac": round(fl / t / PEAK_FLOPS[dkey], 4)}
+    fl = step_flops(cfg, [length] * n_prompts)
+    n = n_prompts * length
+    return {"value": round(n / t, 1), "tokens": n, "ms": round(t * 1e3, 3), "frac": round(fl / t / PEAK_FLOPS[dkey], 4)}
 
 
 def mixed_run(model, cfg, rng, n_req=64, new=128):
@@ -197,13 +199,13 @@ def mixed_run(model, cfg, rng, n_req=64, new=128):
                 requests_equal_in_both_runs=same, requests=n_req, preemptions=model.stats().get("preemptions", 0))
 
 
-def kernel_table(model, cfg, rng, batch, prompt_len):
+def kernel_table(model, cfg, rng, batch, prompt_len, n_prompts=2, length=1024):
     """--profile-stages: every kernel of a prefill step and of a few decode steps timed on the device,
     against the bytes it must move and the flops it must do (stderr)."""
     from deliverance_amd.profiler import KernelProfiler
     KernelProfiler.enable()
-    prefill_run(model, cfg, rng, "bf16")
-    print(KernelProfiler.summary("prefill, 2 x 1,024 tokens, 5 steps (% of 8 TB/s or of the matrix peak, whichever binds)"),
+    prefill_run(model, cfg, rng, "bf16", n_prompts, length)
+    print(KernelProfiler.summary(f"prefill, {n_prompts} x {length:,} tokens, 5 steps (% of 8 TB/s or of the matrix peak, whichever binds)"),
           file=sys.stderr)
     KernelProfiler.reset()
     decode_run(model, cfg, rng, batch, prompt_len, 16, 0)
@@ -228,6 +230,10 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the GPT-2 1.5B points and the 355M mixed workload")
     ap.add_argument("--profile-stages", action="store_true", help="also print a per-kernel table with roofline fractions (stderr)")
+    ap.add_argument("--prefill-shape", default="2x1024", help="prompts x tokens of the prefill step (the contract's: 2x1024)")
+    ap.add_argument("--pool-tokens", type=int, default=None,
+                    help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
+                         "requests out of the cache and back, which the line reports as preemptions)")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="mixed: only the mixed workload, on --model (64 requests with prompts of 16 to 895 tokens arrive at "
                          "once, prompt portions of 512 tokens run beside the decoding of the others, 128 new tokens each)")
@@ -244,12 +250,17 @@ def main():
     el = 2 if args.dtype == "bfloat16" else 4
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     rng = np.random.default_rng(0)
+    pf_n, pf_len = (int(x) for x in args.prefill_shape.lower().split("x"))
+    if not args.no_prefill and args.workload == "decode" and pf_len > cfg["n_positions"]:
+        print(f"a prompt of {pf_len} tokens exceeds n_positions {cfg['n_positions']}")
+        return 2
     if args.prompt_len + SETTLE_STEPS + args.warmup + args.steps + 9 > cfg["n_positions"]:
         print(f"prompt {args.prompt_len} + {SETTLE_STEPS + args.warmup + args.steps + 9} decoded tokens exceed n_positions {cfg['n_positions']}")
         return 2
 
     if args.workload == "mixed":
-        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=512 + 64, max_chunk=512)
+        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=512 + 64, max_chunk=512,
+                                        **({"max_cached_tokens": args.pool_tokens} if args.pool_tokens else {}))
         m = mixed_run(model, cfg, rng)
         print(json.dumps({
             "metric": "generated tok/s, %d requests at once (GPT-2 %s layer sizes, prompts 16..%d, 128 new tokens each, "
@@ -259,13 +270,14 @@ def main():
                 "seconds", "prompt_tokens", "generated_tokens", "all_tokens_per_second", "requests_equal_in_both_runs")},
             "config": {"model": "gpt2-" + args.model, "n_layer": cfg["n_layer"], "n_embd": cfg["n_embd"],
                        "n_head": cfg["n_head"], "requests": m["requests"], "max_chunk": 512, "page_size": 16,
-                       "steps": m["steps"], "mean_batch_tokens": m["mean_batch_tokens"], "preemptions": m["preemptions"]}}))
+                       "steps": m["steps"], "mean_batch_tokens": m["mean_batch_tokens"], "preemptions": m["preemptions"],
+                       "pool_tokens": model.engine_config.max_cached_tokens}}))
         return 0
 
     with tempfile.TemporaryDirectory() as folder:
         random_model(folder, cfg, seed=0)
         model = engine_from_folder(folder, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), cfg,
-                                   kernels=args.kernels)
+                                   kernels=args.kernels, max_batch_tokens=max(2048, args.batch, pf_n * pf_len))
     dt, ctx_mean = decode_run(model, cfg, rng, args.batch, args.prompt_len, args.steps, args.warmup)
     achieved = decode_roofline(cfg, el, args.batch, ctx_mean, dt / args.steps)
     out = {
@@ -289,9 +301,9 @@ def main():
             points[f"decode_b{b}"] = round(b * steps / d, 1)
             fracs[f"decode_b{b}"] = round(decode_roofline(cfg, el, b, cm, d / steps) / HBM_GBS, 4)
     if not args.no_prefill:
-        out["prefill"] = prefill_run(model, cfg, rng, dkey)
+        out["prefill"] = prefill_run(model, cfg, rng, dkey, pf_n, pf_len)
     if args.profile_stages:
-        kernel_table(model, cfg, rng, args.batch, args.prompt_len)
+        kernel_table(model, cfg, rng, args.batch, args.prompt_len, pf_n, pf_len)
     del model
 
     if not args.no_extra and args.dtype == "bfloat16":

@@ -340,9 +340,9 @@ static int decode_launch(const void* q, int q_ld, const void* cache, const int* 
                          const int* seq_lens, int S, int Hq, int Hkv, int D, int page, float scale, int window,
                          void* out, int out_ld, int n_splits, int span, float* partial, hipStream_t st) {
   const int pieces = D / 8;
-  // 8 wavefronts; 16 where the workgroups are few (a context above 512 is then still one chunk a
-  // wavefront, and the larger workgroup's start is paid once per compute unit)
-  const bool wide = (long)S * Hq * n_splits <= 128 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
+  // 8 wavefronts; 16 where the workgroups are no more than the compute units (a context above 512 is then
+  // still one chunk a wavefront, and the larger workgroup's start is paid once per compute unit)
+  const bool wide = (long)S * Hq * n_splits <= 256 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
   dim3 grid(S * Hq, n_splits);
 #define LAUNCH3(C, W, SP)                                                                                   \
   hipLaunchKernelGGL((attn_decode_kernel<C, W, SP>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, \

@@ -70,10 +70,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   bf16_t (*Vs2)[V_TILE] = (bf16_t (*)[V_TILE])(smem + NB * K_TILE * 2);
   __shared__ int bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];
 
-  const int s = seq0 + blockIdx.z, h = blockIdx.y;
+  // The workgroups with the most keys (the last rows) are launched first, those of every (sequence, head) pair
+  // before anybody's second-longest: blockIdx.x, which the dispatcher counts up first, is the pair.  (Counted the
+  // other way round, the long workgroups of the later pairs start when the chip is already full of short ones, and
+  // the step ends with a few compute units walking their keys alone: at 2 x 4,096 rows and 12 heads the wavefronts
+  // resident over the kernel's time averaged 0.9 a SIMD of 2.)
+  const int s = seq0 + (int)blockIdx.x / Hq, h = (int)blockIdx.x % Hq;
   const int row0 = q_start[s], T = q_start[s + 1] - row0;
-  // the workgroups with the most keys (the last rows) are launched first
-  const int i0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * PF_BQ;
+  const int i0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * PF_BQ;
   if (i0 >= T) return;
   const int past = seq_lens[s] - T;
   const int hk = h / (Hq / Hkv);
@@ -200,9 +204,6 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     }
   };
   const int kt0 = (b_lo / (RT * PF_BK)) * (RT * PF_BK);
-  fetch(rk0, rv0, kt0);
-  if (KP == 1 && kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
-
   // the products of one tile, out of LDS buffer `buf`
   auto tile = [&](int kt, int buf) {
     const bf16_t* Ks = Ks2[buf];
@@ -298,15 +299,28 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   // was last read two tiles ago, before the previous barrier.
   if constexpr (KP == 1) {
   int kt = kt0;
-  for (; kt + 4 * PF_BK - 1 <= b_last; kt += 2 * PF_BK) {
-    stash(rk0, rv0, 0);
-    lds_barrier();
-    fetch_fast(rk0, rv0, kt + 2 * PF_BK);
-    tile(kt, 0);
-    stash(rk1, rv1, 1);
-    lds_barrier();
-    fetch_fast(rk1, rv1, kt + 3 * PF_BK);
-    tile(kt + PF_BK, 1);
+  // Where the keys start at a tile's edge (no window, or one that happens to) and the steady state runs
+  // at least once, its first two tiles are asked for the way it asks for all others: the loop is then
+  // entered with the same loads in flight, in the same order, as it is re-entered, and the compiler counts
+  // exactly how many may stay in flight at each wait.  (Entered after the clamping loads it waited for all
+  // of them, and every second tile's keys had one tile's time to arrive instead of two.)  Elsewhere the
+  // loop below, which takes any tile, does all of them.
+  if (b_lo == kt0 && kt0 + 4 * PF_BK - 1 <= b_last) {
+    fetch_fast(rk0, rv0, kt0);
+    fetch_fast(rk1, rv1, kt0 + PF_BK);
+    for (; kt + 4 * PF_BK - 1 <= b_last; kt += 2 * PF_BK) {
+      stash(rk0, rv0, 0);
+      lds_barrier();
+      fetch_fast(rk0, rv0, kt + 2 * PF_BK);
+      tile(kt, 0);
+      stash(rk1, rv1, 1);
+      lds_barrier();
+      fetch_fast(rk1, rv1, kt + 3 * PF_BK);
+      tile(kt + PF_BK, 1);
+    }
+  } else {
+    fetch(rk0, rv0, kt0);
+    if (kt0 + PF_BK <= b_last) fetch(rk1, rv1, kt0 + PF_BK);
   }
   for (int parity = 0; kt <= b_last; kt += PF_BK, parity ^= 1) {
     if (parity == 0) {
@@ -324,6 +338,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     // Key phases: a round parks KP tiles (one register set: the next round's loads fly while this
     // round's tiles are multiplied), each wavefront multiplies the tile of its phase.  Two barriers a
     // round: the tiles are parked before anyone reads them and read before they are replaced.
+    fetch(rk0, rv0, kt0);
     for (int kt = kt0; kt <= b_last; kt += KP * PF_BK) {
       stash(rk0, rv0, 0);
       lds_barrier();
@@ -393,7 +408,7 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
              "attn_prefill: operands must be 16-byte aligned");
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_prefill: bad window or block table");
   DA_REQUIRE(scale > 0.f, "attn_prefill: the score scale must be positive, found %g", (double)scale);
-  DA_REQUIRE(n_seqs <= 65535 && Hq <= 65535, "attn_prefill: too many sequences or heads for one launch");
+  DA_REQUIRE((long)n_seqs * Hq < (1L << 31) && max_query_len <= 65535 * 32, "attn_prefill: too many sequences, heads or rows for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   // The workgroup's form, row blocks x key phases.  Short portions (after a long past, beside decoded
@@ -403,8 +418,12 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   // more than one workgroup a compute unit; else 4 x 1.  Measured on MI355X, head size 64, microseconds
   // 4x1 / 4x2 / 2x2 / 1x4: 2 x 1,024 rows, 12 heads 23.3 / 19.3 / 23.4 / 34.6; 2,048 rows 40.0 / 31.8 /
   // 38.9 / 51.7; 8 x 512 rows 19.3 / 23.3 / 26.2 / 42.5; 4 x 64 rows after 900 keys 22.8 / 17.8 / 17.8 /
-  // 16.3; 16 x 2 rows after 1,000 keys 22.8 / 18.5 / 18.3 / 18.0.  Forms with phases need their tiles in LDS at once: head sizes up
-  // to 64 (4 x 2, 1 x 4) or 128 (2 x 2).  The choice reads the step's shape only.
+  // 16.3; 16 x 2 rows after 1,000 keys 22.8 / 18.5 / 18.3 / 18.0.  With the longest workgroups of every pair launched
+  // first, 4x1 / 4x2: 2 x 1,024 rows, 12 heads 23.2 / 20.0, 25 heads 26.0 / 25.5; 8 x 1,024 rows, 12 heads 35.5 / 39.9;
+  // 2 x 4,096 rows 93.6 / 108.5 (551 TFLOP/s; 157.6 before); 8,192 rows 165.5 / 190.2; 4 x 512 rows after 512 keys,
+  // 16 heads 22.5 / 19.7.  Workgroups of 256 rows (8 x 1) were behind 4 x 1 at every one of these.
+  // Forms with phases need their tiles in LDS at once: head sizes up to 64 (4 x 2, 1 x 4) or 128 (2 x 2).  The
+  // choice reads the step's shape only.
   // form: 0 leaves the choice to this rule; 41, 42, 22 or 14 fixes it
   const long per128 = (long)da_ceil_div(max_query_len, 128) * Hq * n_seqs;
   const int chosen = form ? form
@@ -416,7 +435,7 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   // every key a workgroup can see lies within max_blocks pages
   const bool bt_lds = max_blocks <= (chosen == 41 ? PF_BT_MAX : PF_BT_MAX_PHASED);
 #define LAUNCH2(N, RB, KP, L)                                                                                  \
-  hipLaunchKernelGGL((attn_prefill_kernel<N, RB, KP, L>), dim3(da_ceil_div(max_query_len, 32 * RB), Hq, n_seqs), \
+  hipLaunchKernelGGL((attn_prefill_kernel<N, RB, KP, L>), dim3(Hq * n_seqs, da_ceil_div(max_query_len, 32 * RB)), \
                      dim3(RB * KP * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
                      max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld)
 #define LAUNCH3(N, RB, KP)                \
