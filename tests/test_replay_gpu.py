@@ -97,6 +97,24 @@ def test_cutting_does_not_change_logits_beyond_rounding(model_b, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_neighbours_do_not_change_logits_beyond_rounding(model_b, dtype):
+    """A request alone and the same request beside three others (portions beside decoded tokens, longer and
+    shorter neighbours, which change the attention kernels' forms and the products' row counts): 32-bit sums
+    keep their order whatever shares the step; in bfloat16 the forms that a step takes depend on its shape,
+    so a request's rounding may differ with its neighbours, within the bound that cutting is held to."""
+    m = model_b
+    ids = m.prompt(88, salt=7)
+    alone = helpers.replay(session_for(m, dtype, 128), helpers.trace_bulk_then_single("x", ids, 24))["x"]
+    others = [("n%d" % i, m.prompt(n, salt=20 + i)) for i, n in enumerate((96, 33, 64))]
+    steps = helpers.trace_mixed([("x", ids)] + others, seed=3, max_live=4)
+    s = session_for(m, dtype, helpers.max_live_tokens(steps))
+    beside = helpers.replay(s, steps)["x"]
+    assert beside.shape == alone.shape
+    tol = 1e-6 if dtype == "float32" else 6e-3
+    assert np.abs(beside - alone).max() <= tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(model_a, dtype):
     m = model_a
     ids = m.prompt(128)                       # the whole context, one token a step from the first
