@@ -28,6 +28,8 @@
 // step's shape on the host.  Smaller row blocks are for short portions only: every row block of 32
 // reads its keys anew, and on long prompts that traffic, not the longest workgroup, binds.
 #include "common.h"
+#include <da_lane_swap.h>
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
@@ -42,9 +44,8 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 // for the workgroup's keys fit its LDS copy (a table entry read from memory in front of a tile's loads
 // makes them wait for it, and for every load still in flight)
 template <int D16, int RB, int KP, bool BT_LDS>
-// (head sizes up to 64 with key phases and four wavefronts: registers held to 256, so that two
-// workgroups share a compute unit)
-__global__ void __launch_bounds__(RB * KP * DA_WAVE, (KP > 1 && RB * KP == 4 && D16 <= 4) ? 2 : 1)
+// (head sizes up to 64 with four wavefronts: registers held to 256, so that two workgroups share a compute unit)
+__global__ void __launch_bounds__(RB * KP * DA_WAVE, (RB * KP == 4 && D16 <= 4) ? 2 : 1)
 attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                     const int* __restrict__ block_table, int max_blocks,
                     const int* __restrict__ q_start, const int* __restrict__ seq_lens, int seq0,
@@ -68,7 +69,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES > MERGE_FLOATS * 4 ? TILE_BYTES : MERGE_FLOATS * 4];
   bf16_t (*Ks2)[K_TILE] = (bf16_t (*)[K_TILE])smem;
   bf16_t (*Vs2)[V_TILE] = (bf16_t (*)[V_TILE])(smem + NB * K_TILE * 2);
-  __shared__ int bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];
+  __shared__ long long bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];   // a page's place in the cache, in bytes
 
   // The workgroups with the most keys (the last rows) are launched first, those of every (sequence, head) pair
   // before anybody's second-longest: blockIdx.x, which the dispatcher counts up first, is the pair.  (Counted the
@@ -114,7 +115,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   for (int i = 0; i < DT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
-  float m = -INFINITY, l = 0.f;                 // running maximum (base-2 domain) and sum of weights
+  float m = -INFINITY, l = 0.f;                 // running maximum (base-2 domain); sum of the weights of this lane half's keys
   const float scale2 = scale * 1.4426950408889634f;
 
   // The next tile's keys and values are asked for (into registers) before the current tile is
@@ -125,45 +126,69 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   // from memory in front of every tile would make the tile's loads wait for it, and that wait also
   // drains the loads still in flight for the tiles before.
   const int pg_lo = b_lo >> (31 - __builtin_clz(page)), pg_hi = b_last >> (31 - __builtin_clz(page));
+  const long long page_elems = 2LL * Hkv * page * D;
   if (BT_LDS)
-    for (int i = t; i <= pg_hi - pg_lo; i += THREADS) bts[i] = bt[pg_lo + i];
+    for (int i = t; i <= pg_hi - pg_lo; i += THREADS) bts[i] = bt[pg_lo + i] * page_elems * 2;
   __syncthreads();
-  auto page_of = [&](int key_page) -> long long { return BT_LDS ? bts[key_page - pg_lo] : bt[key_page]; };
+  // where a page's keys and values start, in elements from the cache's start
+  auto page_at = [&](int key_page) -> long long { return BT_LDS ? bts[key_page - pg_lo] / 2 : bt[key_page] * page_elems; };
   // Two register sets: while a tile is multiplied, the loads of the next two are in flight.
   uint4 rk0[NK], rv0[NV], rk1[NK], rv1[NV];
   const int lg = 31 - __builtin_clz(page);              // page is a power of two (checked on the host)
-  const long long page_elems = 2LL * Hkv * page * D;
   const bf16_t* kbase = cache + (long long)hk * page * D;
   const bf16_t* vbase = cache + (long long)(Hkv + hk) * page * D;
   // a tile whose 64 keys all lie in b_lo .. b_last: nothing to clamp, nothing to replace
   // (a fetch covers RT consecutive tiles: key rows kt .. kt + 64 RT - 1; a value piece is 8 keys of
   // one dimension of one tile)
   constexpr int VG = PF_BK / 8, VPT = DT * 32 * VG;       // key groups a tile; value pieces a tile
-  auto fetch_fast = [&](uint4* rk, uint4* rv, int kt) {
+  // A tile starts at a multiple of 64 keys, a page holds 16, 32 or 64: which page of the tile's pages a thread's
+  // piece lies in, and where in that page, never changes.  Both are worked out once; a piece's address is then the
+  // page's place (one read of the table in LDS) plus a constant.
+  const char* kconst[NK];
+  const char* vconst[NV];
+  int kpage[NK], vpage[NV];
 #pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int c0 = t + i * THREADS, c = c0 < K_PIECES ? c0 : 0;
-      const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
-      rk[i] = *(const uint4*)(kbase + page_of(key >> lg) * page_elems + (key & (page - 1)) * D + pc * 8);
-    }
+  for (int i = 0; i < NK; ++i) {
+    const int c0 = t + i * THREADS, c = c0 < K_PIECES ? c0 : 0;
+    const int kr = c / (D / 8), pc = c % (D / 8);
+    kpage[i] = kr >> lg;
+    kconst[i] = (const char*)(kbase + (kr & (page - 1)) * D + pc * 8);
+  }
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
-      const int tl = c / VPT, d = (c % VPT) / VG, g = c % VG, key0 = kt + tl * PF_BK + g * 8;
-      const int ds = d < D ? d : 0;                      // rows of a padded 32-dimension tile repeat dimension 0
-      rv[i] = *(const uint4*)(vbase + page_of(key0 >> lg) * page_elems + ds * page + (key0 & (page - 1)));
-    }
+  for (int i = 0; i < NV; ++i) {
+    const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
+    const int tl = c / VPT, d = (c % VPT) / VG, g = c % VG, k0 = tl * PF_BK + g * 8;
+    const int ds = d < D ? d : 0;                        // rows of a padded 32-dimension tile repeat dimension 0
+    vpage[i] = k0 >> lg;
+    vconst[i] = (const char*)(vbase + ds * page + (k0 & (page - 1)));
+  }
+  auto page_bytes = [&](int key_page) -> long long { return BT_LDS ? bts[key_page - pg_lo] : bt[key_page] * page_elems * 2; };
+  auto fetch_k_fast = [&](uint4* rk, int kt) {
+    const int p0 = kt >> lg;
+#pragma unroll
+    for (int i = 0; i < NK; ++i) rk[i] = *(const uint4*)(kconst[i] + page_bytes(p0 + kpage[i]));
   };
-  auto fetch = [&](uint4* rk, uint4* rv, int kt) {
+  auto fetch_v_fast = [&](uint4* rv, int kt) {
+    const int p0 = kt >> lg;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) rv[i] = *(const uint4*)(vconst[i] + page_bytes(p0 + vpage[i]));
+  };
+  auto fetch_fast = [&](uint4* rk, uint4* rv, int kt) {
+    fetch_k_fast(rk, kt);
+    fetch_v_fast(rv, kt);
+  };
+  auto fetch_k = [&](uint4* rk, int kt) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int c0 = t + i * THREADS, c = c0 < K_PIECES ? c0 : 0;
       const int kr = c / (D / 8), pc = c % (D / 8), key = kt + kr;
       const bool ok = key >= b_lo && key <= b_last;
       const int ks = ok ? key : b_last;
-      rk[i] = *(const uint4*)(kbase + page_of(ks >> lg) * page_elems + (ks & (page - 1)) * D + pc * 8);
+      rk[i] = *(const uint4*)(kbase + page_at(ks >> lg) + (ks & (page - 1)) * D + pc * 8);
       if (!ok) rk[i] = make_uint4(0, 0, 0, 0);
     }
+  };
+  auto fetch_v = [&](uint4* rv, int kt) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c0 = t + i * THREADS, c = c0 < V_PIECES ? c0 : 0;
@@ -171,7 +196,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       const bool ok = d < D && key0 + 7 >= b_lo && key0 <= b_last;
       const int ks = ok ? key0 : (b_last / 8) * 8;
       const int ds = d < D ? d : 0;
-      uint4 v = *(const uint4*)(vbase + page_of(ks >> lg) * page_elems + ds * page + (ks & (page - 1)));
+      uint4 v = *(const uint4*)(vbase + page_at(ks >> lg) + ds * page + (ks & (page - 1)));
       if (!ok) v = make_uint4(0, 0, 0, 0);
       if (key0 < b_lo || key0 + 7 > b_last) {          // rows outside were never written for us
         uint32_t u[4] = {v.x, v.y, v.z, v.w};
@@ -183,13 +208,19 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       rv[i] = v;
     }
   };
+  auto fetch = [&](uint4* rk, uint4* rv, int kt) {
+    fetch_k(rk, kt);
+    fetch_v(rv, kt);
+  };
   // (one phase: the tile goes to buffer `buf`; KP phases: tile k of the fetch goes to buffer k)
-  auto stash = [&](const uint4* rk, const uint4* rv, int buf) {
+  auto stash_k = [&](const uint4* rk, int buf) {
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int c = t + i * THREADS, kr = c / (D / 8), pc = c % (D / 8);
       if (K_PIECES % THREADS == 0 || c < K_PIECES) *(uint4*)&Ks2[buf + kr / PF_BK][(kr % PF_BK) * KLD + pc * 8] = rk[i];
     }
+  };
+  auto stash_v = [&](const uint4* rv, int buf) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = t + i * THREADS, tl = c / VPT, d = (c % VPT) / VG, g = c % VG;
@@ -203,30 +234,38 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       }
     }
   };
+  auto stash = [&](const uint4* rk, const uint4* rv, int buf) {
+    stash_k(rk, buf);
+    stash_v(rv, buf);
+  };
   const int kt0 = (b_lo / (RT * PF_BK)) * (RT * PF_BK);
-  // the products of one tile, out of LDS buffer `buf`
-  auto tile = [&](int kt, int buf) {
+  // The scores of one tile, out of LDS buffer `buf`: S^T = K . Q^T.
+  auto scores = [&](int buf, floatx16 (&sc)[2]) {
     const bf16_t* Ks = Ks2[buf];
-    const bf16_t* Vs = Vs2[buf];
-    if (wave_on && kt <= w_last && kt + PF_BK - 1 >= w_lo) {
-      floatx16 sc[2];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[ks][r] = 0.f;
+      for (int r = 0; r < 16; ++r) sc[ks][r] = 0.f;
 #pragma unroll
-        for (int kd = 0; kd < D16; ++kd) {
-          const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ks[(ks * 32 + col) * KLD + kd * 16 + hf * 8]);
-          sc[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kd], sc[ks], 0, 0, 0);
-        }
+      for (int kd = 0; kd < D16; ++kd) {
+        const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Ks[(ks * 32 + col) * KLD + kd * 16 + hf * 8]);
+        sc[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kd], sc[ks], 0, 0, 0);
       }
+    }
+  };
+  // Mask, running maximum, weights, and the weighted sum of the tile's values out of LDS buffer `buf`.
+  // WHOLE: every row of the wavefront sees all of the tile's keys, known when compiled (no mask, no branch).
+  auto weigh = [&](int kt, int buf, floatx16 (&sc)[2], auto wholec) {
+    constexpr bool WHOLE = decltype(wholec)::value;
+    const bf16_t* Vs = Vs2[buf];
+    {
       // Mask, running maximum and weights.  The maximum is kept in the base-2 domain
       // (s * scale * log2 e, scale > 0), so that a weight costs one multiply-add and one hardware
       // exp2.  A tile that every row of the wavefront sees whole needs no mask at all; elsewhere a key
       // outside q_lo .. pq gets -inf added (0 otherwise), computed from the sign of
       // min(pq - key, key - q_lo) without a comparison: scores are finite, keys that do not exist
       // were loaded as zeros.
-      const bool whole = kt + PF_BK - 1 <= w_first && (window <= 0 || kt >= w_last - window + 1);
+      const bool whole = WHOLE || (kt + PF_BK - 1 <= w_first && (window <= 0 || kt >= w_last - window + 1));
       float tmax = -INFINITY;
       if (whole) {
 #pragma unroll
@@ -248,7 +287,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
             tmax = fmaxf(tmax, v);
           }
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DA_WAVE)) * scale2;
+      tmax = half_max(tmax) * scale2;                  // over both halves of the wavefront: all 64 keys of the row
       const float m_new = fmaxf(m, tmax);
       const bool any = m_new != -INFINITY;             // a row that has seen no key yet keeps zeros
       const float m_use = any ? m_new : 0.f;           // -inf - 0 stays -inf: weight 0, never NaN
@@ -269,11 +308,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           }
           pf[ks][kb] = __builtin_bit_cast(bf16x8_t, make_uint4(u[0], u[1], u[2], u[3]));
         }
-      tsum += __shfl_xor(tsum, 32, DA_WAVE);
-      l = l * alpha + tsum;
+      l = l * alpha + tsum;                            // this half's keys only: the halves' sums meet at the end
       m = m_new;
-      // (skipping this when no row's maximum rose costs a second copy of the output's registers at
-      // the branch, and with it half of the wavefronts a compute unit holds)
+      // (skipping this when no row's maximum rose was measured: no gain, some row of 32 mostly has a new one)
 #pragma unroll
       for (int i = 0; i < DT; ++i)
 #pragma unroll
@@ -289,6 +326,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
             const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&Vs[(i * 32 + col) * PF_VLD + ks * 32 + kb * 16 + 8 * hf]);
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[ks][kb], acc_o[i], 0, 0, 0);
           }
+    }
+  };
+  // the products of one tile, out of LDS buffer `buf`
+  auto tile = [&](int kt, int buf) {
+    if (wave_on && kt <= w_last && kt + PF_BK - 1 >= w_lo) {
+      floatx16 sc[2];
+      scores(buf, sc);
+      weigh(kt, buf, sc, std::false_type{});
     }
   };
 
@@ -349,6 +394,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       lds_barrier();
     }
     // the phases' partial results, merged by phase 0 in the order of the phases
+    l += __shfl_xor(l, 32, DA_WAVE);                    // (both halves had the same maximum all along)
     float* mg = (float*)smem;
     constexpr int PER = DT * 16 + 2;
     if (kp > 0) {
@@ -378,6 +424,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     }
   }
 
+  if constexpr (KP == 1) l += __shfl_xor(l, 32, DA_WAVE);   // (both halves had the same maximum all along)
   if (q_ok) {
     const float inv = 1.0f / l;
     bf16_t* orow = out + (size_t)(row0 + qi) * out_ld + h * D;
@@ -421,7 +468,10 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   // 16.3; 16 x 2 rows after 1,000 keys 22.8 / 18.5 / 18.3 / 18.0.  With the longest workgroups of every pair launched
   // first, 4x1 / 4x2: 2 x 1,024 rows, 12 heads 23.2 / 20.0, 25 heads 26.0 / 25.5; 8 x 1,024 rows, 12 heads 35.5 / 39.9;
   // 2 x 4,096 rows 93.6 / 108.5 (551 TFLOP/s; 157.6 before); 8,192 rows 165.5 / 190.2; 4 x 512 rows after 512 keys,
-  // 16 heads 22.5 / 19.7.  Workgroups of 256 rows (8 x 1) were behind 4 x 1 at every one of these.
+  // 16 heads 22.5 / 19.7.  Workgroups of 256 rows (8 x 1) were behind 4 x 1 at every one of these.  A loop that multiplies
+  // the scores of tile j + 1 while tile j is weighed (keys parked one tile ahead of values) gave the same bits and
+  // -8 % to +12 % of 4 x 1's time depending on the shape: with two wavefronts a SIMD the matrix cores already run under
+  // the other wavefront's softmax; it is not kept.
   // Forms with phases need their tiles in LDS at once: head sizes up to 64 (4 x 2, 1 x 4) or 128 (2 x 2).  The
   // choice reads the step's shape only.
   // form: 0 leaves the choice to this rule; 41, 42, 22 or 14 fixes it
