@@ -471,7 +471,8 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   // 16 heads 22.5 / 19.7.  Workgroups of 256 rows (8 x 1) were behind 4 x 1 at every one of these.  A loop that multiplies
   // the scores of tile j + 1 while tile j is weighed (keys parked one tile ahead of values) gave the same bits and
   // -8 % to +12 % of 4 x 1's time depending on the shape: with two wavefronts a SIMD the matrix cores already run under
-  // the other wavefront's softmax; it is not kept.
+  // the other wavefront's softmax; it is not kept.  Four key phases (2 x 4, 4 x 4) were behind 4 x 2 at every shape (2 x
+  // 1,024 rows, 12 heads: 20.5 and 22.3 against 18.3 us): a round's two barriers and the merge cost more than they share out.
   // Forms with phases need their tiles in LDS at once: head sizes up to 64 (4 x 2, 1 x 4) or 128 (2 x 2).  The
   // choice reads the step's shape only.
   // form: 0 leaves the choice to this rule; 41, 42, 22 or 14 fixes it

@@ -135,13 +135,15 @@ tile_epilogue(floatx16 (&acc)[BM / WM / 32][BN / WN / 32], const float (&bias)[B
     int* slots = (int*)(smem + tile_out_bytes<BM, BN, OUTMODE>());      // the tile rows' places, -1: none
     for (int i = t; i < BM; i += THREADS) slots[i] = m0 + i < M ? kv.slot_map[m0 + i] : -1;
     lds_barrier();
+    // (the page size is a power of two, checked on the host: a place splits into page and row by shift and mask)
+    const int lgp = 31 - __builtin_clz(kv.page), pmask = kv.page - 1;
     const bool kwide = (uintptr_t)kv.cache % 16 == 0 && kv.D % 8 == 0 && kv.q_cols % 8 == 0;
     const int v0 = kv.q_cols + kv.kv_cols;                              // the first value column
 #pragma unroll
     for (int k = 0; k < NCHK; ++k) {
       const int slot = slots[mm[k] - m0];
       if (slot < 0 || nn[k] >= N || nn[k] + 8 <= kv.q_cols || nn[k] >= v0) continue;
-      const int pg = slot / kv.page, prow = slot % kv.page;
+      const int pg = slot >> lgp, prow = slot & pmask;
       if (kwide) {                              // eight dimensions of one key: one piece of its row
         const int c2 = nn[k] - kv.q_cols, h = c2 / kv.D, d = c2 % kv.D;
         *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg, h, prow, kv.Hkv, kv.page, kv.D) + d) = val[k];
@@ -153,35 +155,40 @@ tile_epilogue(floatx16 (&acc)[BM / WM / 32][BN / WN / 32], const float (&bias)[B
         if (nn[k] + e >= kv.q_cols && nn[k] + e < v0)
           kv_scatter_bits(kv, pg, prow, nn[k] + e, (bf16_t)(words[e / 2] >> (16 * (e % 2))));
     }
-    constexpr int NU = (BM / 8) * BN / THREADS;       // (8 rows, column) units a thread; a wavefront's share one row group
-    static_assert((BM / 8) * BN % THREADS == 0 && BN % 64 == 0, "the tile's value units do not split over the threads");
-    const bool vwide = (uintptr_t)kv.cache % 16 == 0 && kv.page % 8 == 0;
+    // Values, straight from the accumulators: a lane holds 4 consecutive rows of its column (r % 4), which are 8
+    // consecutive bytes of the dimension-major page when the rows' places are 4 consecutive ones from a multiple
+    // of 4 on (a prompt portion's are); the lane of the other half holds the 4 rows beside them.
+    const bool vwide = (uintptr_t)kv.cache % 8 == 0 && kv.page % 4 == 0;
+    const long long page_stride = 2LL * kv.Hkv * kv.page * kv.D;
+    bf16_t* vb = (bf16_t*)kv.cache;
 #pragma unroll
-    for (int k = 0; k < NU; ++k) {
-      const int u = t + THREADS * k, g = u / BN, cl = u % BN, n = n0 + cl;
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn + j * 32 + fr;
       if (n < v0 || n >= N) continue;
-      const int cc = n - v0, h = cc / kv.D, d = cc % kv.D;
-      const bf16_t* col = (const bf16_t*)smem + (size_t)(8 * g) * LDT + cl;
-      int sl[8];
-      uint32_t bits[8];
+      const int cc = n - v0;
+      const int vcol = (kv.Hkv + cc / kv.D) * kv.page * kv.D + (cc % kv.D) * kv.page;   // the column's run in a page
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        sl[e] = slots[8 * g + e];
-        bits[e] = col[e * LDT];
-      }
-      bool run = vwide && sl[0] >= 0 && sl[0] % 8 == 0 && sl[0] % kv.page + 7 < kv.page;
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int e = 1; e < 8; ++e) run = run && sl[e] == sl[0] + e;
-      bf16_t* vb = (bf16_t*)kv.cache;
-      if (run) {
-        const uint4 pk = make_uint4(bits[0] | bits[1] << 16, bits[2] | bits[3] << 16, bits[4] | bits[5] << 16, bits[6] | bits[7] << 16);
-        *(uint4*)(vb + cache_v_base(sl[0] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[0] % kv.page) = pk;
-        continue;
-      }
+        for (int q = 0; q < 4; ++q) {
+          const int r0 = wm + i * 32 + 8 * q + 4 * (lane / 32);           // the first of the lane's 4 tile rows
+          const uint4 su = *(const uint4*)&slots[r0];
+          const int s4[4] = {(int)su.x, (int)su.y, (int)su.z, (int)su.w};
+          uint32_t w2[2];
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (sl[e] >= 0)
-          vb[cache_v_base(sl[e] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[e] % kv.page] = (bf16_t)bits[e];
+          for (int e = 0; e < 2; ++e)
+            w2[e] = pack2_bf16(apply_act_bf16(acc[i][j][4 * q + 2 * e] + bias[j], ACT),
+                               apply_act_bf16(acc[i][j][4 * q + 2 * e + 1] + bias[j], ACT));
+          const bool run = vwide && s4[0] >= 0 && (s4[0] & 3) == 0 && s4[1] == s4[0] + 1 && s4[2] == s4[0] + 2 && s4[3] == s4[0] + 3;
+          if (run) {
+            *(uint2*)(vb + (long long)(s4[0] >> lgp) * page_stride + vcol + (s4[0] & pmask)) = make_uint2(w2[0], w2[1]);
+            continue;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (s4[e] >= 0)
+              vb[(long long)(s4[e] >> lgp) * page_stride + vcol + (s4[e] & pmask)] = (bf16_t)(w2[e / 2] >> (16 * (e % 2)));
+        }
     }
   }
 }
@@ -732,7 +739,7 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16: unknown activation %d", act);
   if (kv_cache) {
     DA_REQUIRE(out_dtype == DA_BF16 && !accumulate && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N &&
-               page > 0, "gemm_bf16: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);
+               page > 0 && (page & (page - 1)) == 0, "gemm_bf16: the q|k|v columns (%d + 2*%d) must add up to N=%d, the page size a power of two", q_cols, kv_cols, N);
   }
   if (M == 0) return 0;
   Epilogue ep{bias, bias_dtype, act, accumulate, out, out_dtype, ldo};

@@ -48,6 +48,28 @@ wide_epilogue(floatx16 (&acc)[TM][TN], const float (&bias)[TN], char* region, co
   const int fr = lane % 32;
   int* slots = (int*)(region + 32 * LDT * ES);
   const bool wide = (uintptr_t)ep.out % 16 == 0 && ep.ldo % CH == 0;
+  // A q|k|v product's cache write: what does not change from pass to pass.  The page size is a power of two
+  // (checked on the host): places split into page and row by shift and mask.
+  const int lgp = kv.cache ? 31 - __builtin_clz(kv.page) : 0, pmask = kv.page - 1;
+  const int v0 = kv.q_cols + kv.kv_cols;                        // the first value column
+  const bool kwide = kv.cache && (uintptr_t)kv.cache % 16 == 0 && kv.D % 8 == 0 && kv.q_cols % 8 == 0;
+  const bool vwide = kv.cache && (uintptr_t)kv.cache % 8 == 0 && kv.page % 4 == 0;
+  const long long page_stride = 2LL * kv.Hkv * kv.page * kv.D;
+  int kh[NCHK], kd[NCHK];                                       // head and dimension of a key piece's first column
+  int vcol[TN];                                                 // a value column's place in a page: its head's values, its dimension's run
+  if (OUTMODE == 0 && kv.cache) {
+#pragma unroll
+    for (int k = 0; k < NCHK; ++k) {
+      const int c2 = nw + ((lane + 64 * k) % CPR) * CH - kv.q_cols, cs = c2 > 0 ? c2 : 0;
+      kh[k] = cs / kv.D;
+      kd[k] = cs % kv.D;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int cc = nw + j * 32 + fr - v0, cs = cc > 0 ? cc : 0;
+      vcol[j] = (kv.Hkv + cs / kv.D) * kv.page * kv.D + (cs % kv.D) * kv.page;
+    }
+  }
   // (a pass per constant i: an index that is not a constant would put the accumulators into memory)
   auto pass = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
@@ -110,16 +132,15 @@ wide_epilogue(floatx16 (&acc)[TM][TN], const float (&bias)[TN], char* region, co
     }
 
     if (OUTMODE == 0 && kv.cache) {
-      const bool kwide = (uintptr_t)kv.cache % 16 == 0 && kv.D % 8 == 0 && kv.q_cols % 8 == 0;
-      const int v0 = kv.q_cols + kv.kv_cols;                    // the first value column
+      // keys: eight dimensions of one key are one piece of its cache row (head and dimension of a piece's
+      // columns were worked out before the passes)
 #pragma unroll
       for (int k = 0; k < NCHK; ++k) {
         const int slot = slots[mm[k] - mp];
         if (slot < 0 || nn[k] >= N || nn[k] + 8 <= kv.q_cols || nn[k] >= v0) continue;
-        const int pg = slot / kv.page, prow = slot % kv.page;
-        if (kwide) {                                            // eight dimensions of one key: one piece of its row
-          const int c2 = nn[k] - kv.q_cols, h = c2 / kv.D, d = c2 % kv.D;
-          *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg, h, prow, kv.Hkv, kv.page, kv.D) + d) = val[k];
+        const int pg = slot >> lgp, prow = slot & pmask;
+        if (kwide) {
+          *(uint4*)((bf16_t*)kv.cache + cache_k_row(pg, kh[k], prow, kv.Hkv, kv.page, kv.D) + kd[k]) = val[k];
           continue;
         }
         const uint32_t words[4] = {val[k].x, val[k].y, val[k].z, val[k].w};
@@ -128,38 +149,35 @@ wide_epilogue(floatx16 (&acc)[TM][TN], const float (&bias)[TN], char* region, co
           if (nn[k] + e >= kv.q_cols && nn[k] + e < v0)
             kv_scatter_bits(kv, pg, prow, nn[k] + e, (bf16_t)(words[e / 2] >> (16 * (e % 2))));
       }
-      // values: a lane takes its columns (one of every 64) of each group of 8 rows
-      const bool vwide = (uintptr_t)kv.cache % 16 == 0 && kv.page % 8 == 0;
+      // values, straight from the accumulators: a lane holds 4 consecutive rows of its column (r % 4), which
+      // are 8 consecutive bytes of the dimension-major page when the rows' places are 4 consecutive ones from
+      // a multiple of 4 on (a prompt portion's are); the lane of the other half holds the 4 rows beside them
 #pragma unroll
-      for (int cb = 0; cb < WC; cb += 64) {
-      const int n = nw + cb + lane;
-      if (n >= v0 && n < N) {
-        const int cc = n - v0, h = cc / kv.D, d = cc % kv.D;
+      for (int j = 0; j < TN; ++j) {
+        const int n = nw + j * 32 + fr;
+        if (n < v0 || n >= N) continue;
         bf16_t* vb = (bf16_t*)kv.cache;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const bf16_t* col = (const bf16_t*)region + (size_t)(8 * g) * LDT + cb + lane;
-          int sl[8];
-          uint32_t bits[8];
+        for (int q = 0; q < 4; ++q) {
+          const int r0 = 8 * q + 4 * (lane / 32);             // the first of the lane's 4 rows in this pass
+          const uint4 su = *(const uint4*)&slots[r0];
+          const struct { int x, y, z, w; } sl = {(int)su.x, (int)su.y, (int)su.z, (int)su.w};
+          uint32_t w2[2];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            sl[e] = slots[8 * g + e];
-            bits[e] = col[e * LDT];
-          }
-          bool run = vwide && sl[0] >= 0 && sl[0] % 8 == 0 && sl[0] % kv.page + 7 < kv.page;
-#pragma unroll
-          for (int e = 1; e < 8; ++e) run = run && sl[e] == sl[0] + e;
+          for (int e = 0; e < 2; ++e)
+            w2[e] = pack2_bf16(apply_act_bf16(acc[i][j][4 * q + 2 * e] + bias[j], ACT),
+                               apply_act_bf16(acc[i][j][4 * q + 2 * e + 1] + bias[j], ACT));
+          const bool run = vwide && sl.x >= 0 && (sl.x & 3) == 0 && sl.y == sl.x + 1 && sl.z == sl.x + 2 && sl.w == sl.x + 3;
           if (run) {
-            const uint4 pk = make_uint4(bits[0] | bits[1] << 16, bits[2] | bits[3] << 16, bits[4] | bits[5] << 16, bits[6] | bits[7] << 16);
-            *(uint4*)(vb + cache_v_base(sl[0] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[0] % kv.page) = pk;
+            *(uint2*)(vb + (long long)(sl.x >> lgp) * page_stride + vcol[j] + (sl.x & pmask)) = make_uint2(w2[0], w2[1]);
             continue;
           }
+          const int s4[4] = {sl.x, sl.y, sl.z, sl.w};
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (sl[e] >= 0)
-              vb[cache_v_base(sl[e] / kv.page, h, kv.Hkv, kv.page, kv.D) + (long long)d * kv.page + sl[e] % kv.page] = (bf16_t)bits[e];
+          for (int e = 0; e < 4; ++e)
+            if (s4[e] >= 0)
+              vb[(long long)(s4[e] >> lgp) * page_stride + vcol[j] + (s4[e] & pmask)] = (bf16_t)(w2[e / 2] >> (16 * (e % 2)));
         }
-      }
       }
     }
     wave_lds_sync();       // the next pass parks over what this one read
@@ -426,7 +444,7 @@ extern "C" int da_gemm_bf16_wide(const void* a, int lda, const void* w, int ldw,
              "gemm_bf16_wide: K=%d must be a multiple of %d, and an activation goes with a bfloat16 result", K, WD_BK);
   if (kv_cache) {
     DA_REQUIRE(out_dtype == DA_BF16 && !accumulate && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N &&
-               page > 0, "gemm_bf16_wide: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);
+               page > 0 && (page & (page - 1)) == 0, "gemm_bf16_wide: the q|k|v columns (%d + 2*%d) must add up to N=%d, the page size a power of two", q_cols, kv_cols, N);
   }
   Epilogue ep{bias, bias_dtype, act, accumulate, out, out_dtype, ldo};
   KvScatter kv{kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page};
