@@ -192,7 +192,10 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
 // share a compute unit and N / 16 workgroups run side by side.
 // ---------------------------------------------------------------------------------------------
 #define FL_LD (64 + 8)       // padded row of a parked step of w, elements
-template <int RV, bool PBF16, bool TWO_ROWS>
+// CG: groups of 16 columns a workgroup (one after the other; the rows are normalised once for all of them: with a
+// wide K that work, done again by every workgroup, is what the fused kernel costs, and CG workgroups' worth of it
+// is saved; the next group's loads of w are asked for before this group is multiplied).
+template <int RV, bool PBF16, bool TWO_ROWS, int CG = 1>
 __global__ void __launch_bounds__(512)
 gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilogue ep, KvScatter kv,
                    int M, int N, int K) {
@@ -206,7 +209,8 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
   bf16_t (*stage)[16 * FL_LD] = (bf16_t (*)[16 * FL_LD])stage_red;
   float (*red)[16][FZ_COLS + 1] = (float (*)[16][FZ_COLS + 1])stage_red;
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
-  const int n0 = blockIdx.x * FZ_COLS;
+  const int n_first = blockIdx.x * (FZ_COLS * CG);   // the workgroup's first column
+  int n0 = n_first;                                  // the current group's first column
   const int fr = lane % 16, fk = (lane / 16) * 8;    // a fragment: row fr of 16, k-group lane / 16
   const int lr = lane / 8, lc = (lane % 8) * 8;      // a load of w: row lr of 8, 16-byte piece lane % 8
 
@@ -241,25 +245,30 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
       bq[i] = *(const uint4*)((const float*)(ln.b ? ln.b : ln.g) + cs);
     }
   }
-  // this thread's output element (16 x 16 of them), with what its epilogue needs
-  const int em = t / FZ_COLS, ec = t % FZ_COLS, en = n0 + ec;
-  const bool e_ok = t < 16 * FZ_COLS && em < M && en < N;
-  const int ebn = e_ok ? en : 0;
+  // this thread's output element (16 x 16 of them) of a group, with what its epilogue needs
+  const int em = t / FZ_COLS, ec = t % FZ_COLS;
   const void* e_bsrc = ep.bias ? ep.bias : (const void*)w;
-  const int e_bidx = ep.bias ? ebn : 0;
-  const uint32_t e_bias_raw = PBF16 ? (uint32_t)((const bf16_t*)e_bsrc)[e_bidx] : ((const uint32_t*)e_bsrc)[e_bidx];
-  const int e_slot = kv.cache ? kv.slot_map[e_ok ? em : 0] : -1;
-  uint4 wv[SW][2];
+  const int e_slot = kv.cache ? kv.slot_map[(t < 16 * FZ_COLS && em < M) ? em : 0] : -1;
+  auto bias_bits = [&](int nfirst) -> uint32_t {
+    const int en = nfirst + ec;
+    const int e_bidx = (ep.bias && t < 16 * FZ_COLS && em < M && en < N) ? en : 0;
+    return PBF16 ? (uint32_t)((const bf16_t*)e_bsrc)[e_bidx] : ((const uint32_t*)e_bsrc)[e_bidx];
+  };
+  auto ask_w = [&](uint4 (&wr)[SW][2], int nfirst) {
 #pragma unroll
-  for (int u = 0; u < SW; ++u) {
-    const int k0 = (wave + u * NW) * 64;
-    const int kk = k0 + lc < K ? k0 + lc : 0;        // past K: the row's first piece
+    for (int u = 0; u < SW; ++u) {
+      const int k0 = (wave + u * NW) * 64;
+      const int kk = k0 + lc < K ? k0 + lc : 0;      // past K: the row's first piece
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int n = n0 + i * 8 + lr;
-      wv[u][i] = load16(w + (size_t)(n < N ? n : 0) * ldw + kk);
+      for (int i = 0; i < 2; ++i) {
+        const int n = nfirst + i * 8 + lr;
+        wr[u][i] = load16(w + (size_t)(n < N ? n : 0) * ldw + kk);
+      }
     }
-  }
+  };
+  uint32_t e_bias_raw = bias_bits(n0);
+  uint4 wv[SW][2];
+  ask_w(wv, n0);
   __builtin_amdgcn_sched_barrier(0);                 // the loads stay in this order, ahead of the arithmetic
 
   // ---- statistics and the normalised rows
@@ -312,38 +321,59 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
 
   // ---- products: a step of w is parked, then both operands' fragments come out of LDS
   bf16_t* mine = stage[wave];
-  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int u = 0; u < SW; ++u) {
-    const int k0 = (wave + u * NW) * 64;             // < KMAX: the rows of a are zero from K on
-#pragma unroll
-    for (int i = 0; i < 2; ++i) *(uint4*)&mine[(i * 8 + lr) * FL_LD + lc] = wv[u][i];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    if (SW * NW * 64 <= KMAX || k0 < KMAX) {
-#pragma unroll
-      for (int c = 0; c < 64; c += 32) {
-        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[fr * FL_LD + c + fk]);
-        const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&a_lds[fr % AR][k0 + c + fk]);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc, 0, 0, 0);
-      }
+#pragma unroll 1
+  for (int g = 0; g < CG; ++g) {
+    // the next group's w (and bias) travel while this group is multiplied
+    uint4 wn[SW][2];
+    uint32_t e_bias_next = 0;
+    const bool more = CG > 1 && g + 1 < CG && n0 + FZ_COLS < N;
+    if (CG > 1 && more) {
+      ask_w(wn, n0 + FZ_COLS);
+      e_bias_next = bias_bits(n0 + FZ_COLS);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-  }
-  lds_barrier();                                     // every wavefront is done with its parked steps
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int r = 0; r < 4; ++r) red[wave][4 * (lane / 16) + r][fr] = acc[r];
-  lds_barrier();
-  if (e_ok) {
-    float v = red[0][em][ec];
+    for (int u = 0; u < SW; ++u) {
+      const int k0 = (wave + u * NW) * 64;             // < KMAX: the rows of a are zero from K on
 #pragma unroll
-    for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
-    const float e_bias = !ep.bias ? 0.f : (PBF16 ? __uint_as_float(e_bias_raw << 16) : __uint_as_float(e_bias_raw));
-    epilogue_store(ep, em, en, v, e_bias);
-    if (kv.cache && en >= kv.q_cols && e_slot >= 0) kv_scatter_store(kv, e_slot, en, apply_act_bf16(v + e_bias, ep.act));
+      for (int i = 0; i < 2; ++i) *(uint4*)&mine[(i * 8 + lr) * FL_LD + lc] = wv[u][i];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+      if (SW * NW * 64 <= KMAX || k0 < KMAX) {
+#pragma unroll
+        for (int c = 0; c < 64; c += 32) {
+          const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, *(const uint4*)&mine[fr * FL_LD + c + fk]);
+          const bf16x8_t af = __builtin_bit_cast(bf16x8_t, *(const uint4*)&a_lds[fr % AR][k0 + c + fk]);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc, 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+    lds_barrier();                                     // every wavefront is done with its parked steps
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][4 * (lane / 16) + r][fr] = acc[r];
+    lds_barrier();
+    const int en = n0 + ec;
+    if (t < 16 * FZ_COLS && em < M && en < N) {
+      float v = red[0][em][ec];
+#pragma unroll
+      for (int v2 = 1; v2 < NW; ++v2) v += red[v2][em][ec];
+      const float e_bias = !ep.bias ? 0.f : (PBF16 ? __uint_as_float(e_bias_raw << 16) : __uint_as_float(e_bias_raw));
+      epilogue_store(ep, em, en, v, e_bias);
+      if (kv.cache && en >= kv.q_cols && e_slot >= 0) kv_scatter_store(kv, e_slot, en, apply_act_bf16(v + e_bias, ep.act));
+    }
+    if (CG == 1 || !more) break;
+    lds_barrier();                                     // the sums are read before the next group parks over them
+    n0 += FZ_COLS;
+    e_bias_raw = e_bias_next;
+#pragma unroll
+    for (int u = 0; u < SW; ++u) {
+      wv[u][0] = wn[u][0];
+      wv[u][1] = wn[u][1];
+    }
   }
 }
 
@@ -377,11 +407,18 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
   const int mt = da_ceil_div(M, 16);
   hipStream_t s = (hipStream_t)stream;
   // the kernel with whole-line loads takes one row tile, K up to 2048, and parameters of one dtype
+  // Groups of 16 columns a workgroup.  Measured on MI355X with cold weights, K = 1,600, N = 4,800 and 6,400, against
+  // the norm and the product as two kernels (9.6 to 10.2 us): one group 7.9 to 8.0 us with one row, 8.4 to 8.5 with
+  // 4, 10.1 with 8; two groups 8.0 to 8.2 / 7.9 to 8.5 / 9.1 to 9.6; four groups 11.8 to 13.5 (too few workgroups
+  // pull on memory).  Two from 5 rows on where K is wide.
+  const int groups = (M > 4 && K > 1280) ? 2 : 1;
   const int pdt = g_dtype;
   const bool same = (!b || b_dtype == pdt) && (!bias || bias_dtype == pdt) && (pdt == DA_BF16 || pdt == DA_F32);
 #define LAUNCH_LDS_P(RV, PB)                                                                                      \
   do {                                                                                                            \
-    if (M <= 8)                                                                                                   \
+    if (M <= 8 && RV >= 6 && groups == 2)                                                                    \
+      hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, PB, false, (RV >= 6 ? 2 : 1)>), dim3(da_ceil_div(N, FZ_COLS * 2)), dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
+    else if (M <= 8)                                                                                              \
       hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, PB, false>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \
     else                                                                                                          \
       hipLaunchKernelGGL((gemm_ln_rows_kernel<RV, PB, true>), grid, dim3(512), 0, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K); \

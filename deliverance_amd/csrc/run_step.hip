@@ -39,11 +39,11 @@ extern "C" int da_decode_splits(int n_seqs, int n_heads, int max_blocks, int pag
 
 // Measured on MI355X inside the model: the fused norm + product kernel wins up to 16 rows (one row tile)
 // and a width of 1,024, by 10 to 15 % of a decode step; up to 8 rows (which take half the LDS, so that the
-// workgroups still run side by side) up to a width of 1,280, and a single row up to 2,048; beyond, the
-// separate norm and product are faster (every 16 output columns read and normalise all rows again: at a
-// width of 1,600 and 8 rows 8.0 us against 3.1 + 3.9).  Never for a vocabulary.
+// workgroups still run side by side) up to a width of 2,048: up to 1,280 with 16 columns a workgroup, beyond
+// with 32 from 5 rows on (every workgroup reads and normalises all rows again, and at a width of 1,600 that is
+// 2.5 us of vector work a compute unit; with 32 columns half as many workgroups do it).  Never for a vocabulary.
 extern "C" int da_can_fuse_ln(int n_rows, int K, int N) {
-  const bool fits = (n_rows <= 16 && K <= 1024) || (n_rows <= 8 && K <= 1280) || (n_rows <= 1 && K <= 2048);
+  const bool fits = (n_rows <= 16 && K <= 1024) || (n_rows <= 8 && K <= 2048);
   return n_rows > 0 && fits && K % 8 == 0 && N <= 16384;
 }
 

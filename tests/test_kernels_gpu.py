@@ -719,15 +719,17 @@ def test_product_writes_keys_and_values(ops, M):
 
 
 @pytest.mark.simt_quick
-def test_fused_norm_product_writes_keys_and_values(ops):
+@pytest.mark.parametrize("M,K", [(9, 96), (7, 1312)])
+def test_fused_norm_product_writes_keys_and_values(ops, M, K):
+    """(7 rows and a wide K: two groups of 16 columns a workgroup)"""
     g = torch.Generator().manual_seed(11)
-    Hq, Hkv, D, page, M, K = 6, 2, 48, 16, 9, 96
+    Hq, Hkv, D, page = 6, 2, 48, 16
     N = (Hq + 2 * Hkv) * D
     x = torch.randn(M, K, generator=g).to(DEV)
     gw, gb = bf(torch.randn(K, generator=g)).to(DEV), bf(torch.randn(K, generator=g)).to(DEV)
     w = bf(torch.randn(N, K, generator=g) * 0.1).to(DEV)
     bias = bf(torch.randn(N, generator=g)).to(DEV)
-    slots = torch.tensor([3 * page + 5, -1, 0, 17, 40, 41, 42, 95, 64], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([3 * page + 5, -1, 0, 17, 40, 41, 42, 95, 64][:M], dtype=torch.int32, device=DEV)
     c1 = torch.zeros(6, 2, Hkv, page, D, dtype=torch.bfloat16, device=DEV)
     c2 = torch.zeros_like(c1)
     out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
