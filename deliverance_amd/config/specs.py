@@ -71,7 +71,10 @@ class LayerSpec:
 
     The reference's block has five optional norm places
     (core/.../generator/TransformerBlock.java:26-32); the pre-norm pair is what its
-    GPT-2 uses (TransformerBlock.java:35-41).
+    GPT-2 uses (TransformerBlock.java:35-41).  ``post_block_norm`` is the fifth (applied to
+    the stream when both parts have joined it, TransformerBlock.java:199);
+    ``residual_multiplier`` scales a part's output (after the norm behind it, if any) before
+    it joins the stream (TransformerBlock.java:260-272; 1: plain addition).
     """
     mixer: object
     feed_forward: object
@@ -80,6 +83,8 @@ class LayerSpec:
     pre_ff_norm: Optional[NormSpec] = None
     post_ff_norm: Optional[NormSpec] = None
     weight_prefix: str = ""
+    post_block_norm: Optional[NormSpec] = None
+    residual_multiplier: float = 1.0
 
 
 @dataclass(frozen=True)

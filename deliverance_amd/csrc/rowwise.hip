@@ -46,29 +46,30 @@ extern "C" int da_embed(const int* tokens, const int* positions, const void* wte
 }
 
 // ------------------------------------------------------------------------------------------
-// dst[r, :] (+)= src[rows ? rows[r] : r, :]: rows gathered, converted between 32-bit and
+// dst[r, :] (+)= scale * src[rows ? rows[r] : r, :]: rows gathered, converted between 32-bit and
 // bfloat16, or added into the 32-bit residual stream.  For blocks without a norm in front of a
-// part, models without a final norm, and norms that follow a part.
+// part, models without a final norm, norms that follow a part, and a part's output that joins the
+// stream times a constant (TransformerBlock.java:260-272).
 // ------------------------------------------------------------------------------------------
 __global__ void copy_rows_kernel(const void* __restrict__ src, int src_dtype, const int* __restrict__ rows,
-                                 void* __restrict__ dst, int dst_dtype, int E, int accumulate) {
+                                 void* __restrict__ dst, int dst_dtype, int E, int accumulate, float scale) {
   const int r = blockIdx.x;
   const size_t srow = (size_t)(rows ? rows[r] : r) * E, drow = (size_t)r * E;
   for (int i = threadIdx.x; i < E; i += blockDim.x) {
-    const float v = load_param(src, src_dtype, srow + i);
+    const float v = load_param(src, src_dtype, srow + i) * scale;
     if (accumulate) ((float*)dst)[drow + i] += v;
     else store_out(dst, dst_dtype, drow + i, v);
   }
 }
 
 extern "C" int da_copy_rows(const void* src, int src_dtype, const int* rows, void* dst, int dst_dtype, int R,
-                            int E, int accumulate, void* stream) {
+                            int E, int accumulate, float scale, void* stream) {
   DA_REQUIRE(R >= 0 && E > 0, "copy_rows: bad sizes R=%d E=%d", R, E);
   DA_REQUIRE(!accumulate || dst_dtype == DA_F32, "copy_rows: accumulation needs a 32-bit destination");
   if (R == 0) return 0;
   const int threads = E >= 256 ? 256 : (E >= 128 ? 128 : 64);
   hipLaunchKernelGGL(copy_rows_kernel, dim3(R), dim3(threads), 0, (hipStream_t)stream, src, src_dtype, rows, dst,
-                     dst_dtype, E, accumulate);
+                     dst_dtype, E, accumulate, scale);
   DA_CHECK_LAUNCH("copy_rows");
   return 0;
 }

@@ -120,7 +120,8 @@ class NativeStep:
             at, ff = blk.mixer, blk.feed_forward
             if type(at) is not CausalSelfAttention or at.position is not None or at.head_dim % 16 or at.head_dim > 256:
                 return False
-            if type(blk.pre_mixer_norm) is not LayerNorm or blk.post_mixer_norm is not None or blk.post_ff_norm is not None:
+            if (type(blk.pre_mixer_norm) is not LayerNorm or blk.post_mixer_norm is not None or blk.post_ff_norm is not None
+                    or blk.post_block_norm is not None or blk.residual_multiplier != 1.0):
                 return False
             if ff is not None and (type(ff) is not DenseFeedForward or type(blk.pre_ff_norm) is not LayerNorm or ff.inner % 8):
                 return False

@@ -68,7 +68,7 @@ def _check(rc: int):
 _VP, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 _ARGTYPES = {
     "da_embed": [_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _F, _VP],
-    "da_copy_rows": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP],
+    "da_copy_rows": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _F, _VP],
     "da_take_tokens": [_VP, _VP, _VP, _I, _I, _I, _VP],
     "da_fill_zero": [_VP, ctypes.c_long, _VP],
     "da_state_gather": [_VP, _VP, _VP, _VP, _I, _I, _I, _VP],
@@ -163,8 +163,8 @@ def embed(tokens: torch.Tensor, positions: torch.Tensor, wte: torch.Tensor,
 
 
 def copy_rows(src: torch.Tensor, dst: torch.Tensor, rows: Optional[torch.Tensor] = None,
-              accumulate: bool = False) -> torch.Tensor:
-    """dst[r] (+)= src[rows[r]] (or src[r]); 32-bit and bfloat16 on either side, += into 32-bit."""
+              accumulate: bool = False, scale: float = 1.0) -> torch.Tensor:
+    """dst[r] (+)= scale * src[rows[r]] (or src[r]); 32-bit and bfloat16 on either side, += into 32-bit."""
     _dev(src, dst, rows)
     _need(src.dim() == 2 and dst.dim() == 2 and src.is_contiguous() and dst.is_contiguous() and
           src.shape[1] == dst.shape[1], "copy_rows: contiguous matrices of one width are needed")
@@ -175,7 +175,7 @@ def copy_rows(src: torch.Tensor, dst: torch.Tensor, rows: Optional[torch.Tensor]
         _need(rows.dtype == torch.int32 and rows.numel() >= R, "copy_rows: rows must be int32 with a row each")
     _need(not accumulate or dst.dtype == torch.float32, "copy_rows: accumulation needs a float32 destination")
     _check(_lib().da_copy_rows(_ptr(src), _dt(src), _ptr(rows), _ptr(dst), _dt(dst), R, dst.shape[1],
-                               int(accumulate), _stream()))
+                               int(accumulate), float(scale), _stream()))
     return dst
 
 

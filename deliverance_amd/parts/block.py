@@ -2,7 +2,8 @@
 adding into the 32-bit residual stream.
 Reference: core/src/main/java/io/teknek/deliverance/generator/TransformerBlock.java:161-200
 (five optional norm places :26-32; GPT-2 uses the two pre-norms :35-41; a norm after a part acts
-on the part's output before the residual add :172-176,184-188)."""
+on the part's output before the residual add :172-176,184-188; the part's output may join the stream
+times a constant :260-272; the fifth norm acts on the stream at the block's end :199)."""
 from __future__ import annotations
 
 import torch
@@ -20,6 +21,8 @@ class Block:
         self.post_mixer_norm = norm(spec.post_mixer_norm, "post_mixer_norm")
         self.pre_ff_norm = norm(spec.pre_ff_norm, "pre_ff_norm")
         self.post_ff_norm = norm(spec.post_ff_norm, "post_ff_norm")
+        self.post_block_norm = norm(getattr(spec, "post_block_norm", None), "post_block_norm")
+        self.residual_multiplier = float(getattr(spec, "residual_multiplier", 1.0))
         self.mixer = build_mixer(spec.mixer, params["mixer"], dtype, device)
         self.feed_forward = None if spec.feed_forward is None else \
             build_feed_forward(spec.feed_forward, params["feed_forward"], dtype, device)
@@ -31,22 +34,23 @@ class Block:
         h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)      # no norm in front: the stream, converted
         return ops.copy_rows(x, h)
 
-    @staticmethod
-    def _part(ctx, x, pre, post, run, run_normed):
+    def _part(self, ctx, x, pre, post, run, run_normed):
         """One part of the block.  Parts add into the tensor they are given.  Without a norm behind
-        the part that tensor is the residual stream; with one, the part adds into a buffer of its
-        own (cleared by a fill kernel of the engine's, so that a recorded step holds no memset), whose
-        norm, kept in 32-bit, is then added to the stream."""
+        the part (and without a multiplier) that tensor is the residual stream; else the part adds
+        into a buffer of its own (cleared by a fill kernel of the engine's, so that a recorded step
+        holds no memset), whose norm, kept in 32-bit, times the multiplier is then added to the stream."""
         target = x
-        if post is not None:
+        own = post is not None or self.residual_multiplier != 1.0
+        if own:
             target = ops.fill_zero(ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32))
         # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
         # of it itself (fused into its first product) and returns True, or returns False to
         # decline this step.  That needs the part's input and the tensor it adds into to be the same.
-        if not (post is None and pre is not None and run_normed is not None and run_normed(pre)):
+        if not (not own and pre is not None and run_normed is not None and run_normed(pre)):
             run(Block._normed(ctx, x, pre), target)
-        if post is not None:
-            ops.copy_rows(post.forward(ctx, target, out_name="post_norm", out_dtype=torch.float32), x, accumulate=True)
+        if own:
+            out = target if post is None else post.forward(ctx, target, out_name="post_norm", out_dtype=torch.float32)
+            ops.copy_rows(out, x, accumulate=True, scale=self.residual_multiplier)
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
         fused = getattr(self.mixer, "forward_normed", None)
@@ -62,3 +66,5 @@ class Block:
                        None if fused is None else (lambda norm: fused(ctx, norm, x)))
             if ctx.debug_hook is not None:
                 ctx.emit(call.layer, "post_ff_residual", x)
+        if self.post_block_norm is not None:                # the stream itself, normalised in place
+            ops.copy_rows(self.post_block_norm.forward(ctx, x, out_name="post_norm", out_dtype=torch.float32), x)

@@ -198,6 +198,54 @@ def test_block_part_and_fused_small_steps(model_b, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("post", [False, True])
+def test_block_with_a_residual_multiplier_and_a_norm_at_its_end(model_b, dtype, post):
+    """The reference's residual multiplier (TransformerBlock.java:260-272: a part's output, after the norm
+    behind it if there is one, joins the stream times a constant) and its fifth norm place (:199: the stream
+    is normalised when both parts have joined it):
+        x1 = x + c * Attn(N(x));  x2 = x1 + c * MLP(N'(x1));  out = N_end(x2)."""
+    import dataclasses
+    from deliverance_amd.config import Gpt2Config, LayerCall
+    from deliverance_amd.models import gpt2 as arch
+    from deliverance_amd.parts import Block
+    from deliverance_amd.weights import load_declared
+    mc = Gpt2Config.from_dict(helpers.CONFIG_B).to_model_config()
+    bound = arch.bind_tensors(mc, load_declared(model_b.folder, arch.declare_tensors(mc)))
+    layer, W, cfg, c = 1, model_b.W, model_b.plain_cfg, 0.37
+    spec = mc.layers[layer]
+    norm = spec.pre_mixer_norm
+    spec = dataclasses.replace(spec, residual_multiplier=c, post_block_norm=norm, post_mixer_norm=norm if post else None)
+    params = dict(bound["layers"][layer])
+    for key, name in (("post_block_norm", "h.2.ln_2"), ("post_mixer_norm", "h.0.ln_1")):
+        params[key] = {"weight": torch.from_numpy(W[name + ".weight"]).to(torch.bfloat16),
+                       "bias": torch.from_numpy(W[name + ".bias"]).to(torch.bfloat16)}
+    blk = Block(spec, params, dtype, DEV)
+    eps = cfg["layer_norm_epsilon"]
+    H, E = cfg["n_head"], cfg["n_embd"]
+    scale = 1.0 / math.sqrt(E // H) / (layer + 1)
+    g = torch.Generator().manual_seed(8)
+    for T in (33, 3):
+        x0 = torch.randn(T, E, generator=g)
+        ctx = make_ctx(dtype, [T], [0], 2, 48)
+        x = x0.clone().to(DEV)
+        blk.forward(ctx, x, LayerCall(layer, 0, True))
+        xn = x0.double().numpy()
+        o = P.attention_block(P.layer_norm(xn, W[f"h.{layer}.ln_1.weight"], W[f"h.{layer}.ln_1.bias"], eps), W, layer, H, scale)
+        if post:
+            o = P.layer_norm(o, W["h.0.ln_1.weight"], W["h.0.ln_1.bias"], eps)
+        x1 = xn + c * o
+        f = P.mlp_block(P.layer_norm(x1, W[f"h.{layer}.ln_2.weight"], W[f"h.{layer}.ln_2.bias"], eps), W, layer,
+                        cfg["activation_function"])
+        x2 = x1 + c * f
+        want = P.layer_norm(x2, W["h.2.ln_2.weight"], W["h.2.ln_2.bias"], eps)
+        tol = {torch.float32: 2e-4, torch.bfloat16: 1.5e-1 if post else 3e-2}[dtype]
+        assert np.abs(x.double().cpu().numpy() - want).max() < tol, (T, post)
+        plain_sum = P.layer_norm(xn + o + f, W["h.2.ln_2.weight"], W["h.2.ln_2.bias"], eps)
+        if post:
+            assert np.abs(want - plain_sum).max() > 0.1       # (a block that forgot the multiplier is far off)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("pre", [True, False])
 def test_block_with_norms_behind_its_parts(model_b, dtype, pre):
     """The block's other norm places (TransformerBlock.java:26-32,172-176,184-188): a norm behind a
