@@ -116,6 +116,8 @@ class ModelConfig:
     eos_token_ids: Tuple[int, ...]
     raw: dict = field(default_factory=dict, compare=False, hash=False)
     embed_scale: float = 1.0        # multiplies the token embedding before positions are added
+    # logits are divided by it (the reference's logitMultiplier, AbstractGeneratorSampler.java:117-120)
+    logit_multiplier: float = 1.0
 
     @property
     def n_cache_slots(self) -> int:

@@ -112,7 +112,7 @@ class NativeStep:
         if model.device.type != "cuda":
             return False
         cfg = model.config
-        if cfg.width % 8 or type(model.final_norm) is not LayerNorm or model.head_weight.dtype != torch.bfloat16:
+        if cfg.width % 8 or type(model.final_norm) is not LayerNorm or model.head_weight.dtype != torch.bfloat16 or cfg.logit_multiplier != 1.0:
             return False
         if type(model.embed_position) not in (LearnedPositions, NoPositions):
             return False

@@ -95,12 +95,15 @@ class CausalLM:
         ln = None if self.final_norm is None else self.final_norm.fusable_params()
         if ln is not None and ops.can_fuse_ln(n_want, x, self.head_weight):
             gain, bias, eps = ln                   # few wanted rows: norm and head in one kernel
-            return ops.linear_ln(x, want_rows, n_want, gain, bias, eps, self.head_weight, None, logits)
-        if self.final_norm is not None:
-            e = self.final_norm.forward(ctx, x, rows=want_rows, n_rows=n_want, out_name="final_norm")
+            ops.linear_ln(x, want_rows, n_want, gain, bias, eps, self.head_weight, None, logits)
         else:
-            e = ops.copy_rows(x, ctx.buf("final_norm", n_want, self.config.width, ctx.dtype), rows=want_rows)
-        ops.linear(e, self.head_weight, None, logits)
+            if self.final_norm is not None:
+                e = self.final_norm.forward(ctx, x, rows=want_rows, n_rows=n_want, out_name="final_norm")
+            else:
+                e = ops.copy_rows(x, ctx.buf("final_norm", n_want, self.config.width, ctx.dtype), rows=want_rows)
+            ops.linear(e, self.head_weight, None, logits)
+        if self.config.logit_multiplier != 1.0:     # (an architecture's constant; GPT-2 has none)
+            ops.copy_rows(logits, logits, scale=1.0 / self.config.logit_multiplier)
         return logits
 
 

@@ -23,6 +23,7 @@ H0, HKV0, D0, WINDOW, BASE = 6, 2, 16, 24, 100.0     # layer 0: grouped heads, a
 H1, HKV1, D1 = 3, 1, 32                              # layer 1: one key head, every earlier key
 INNER0, INNER_X, N_EXPERTS = 80, 48, 2
 EPS = 1e-6
+LOGIT_MULT = 2.5     # the logits are divided by it (an architecture's constant)
 MARGIN = 0.05        # rows whose router logits lie closer than this are left out of the bfloat16 comparison
 
 
@@ -93,7 +94,7 @@ def _register_once():
         layers = (LayerSpec(a0, DenseFeedForwardSpec("dense", E, INNER0, "relu"), norm, None, norm, None, "l0."),
                   LayerSpec(a1, RoutedSpec("toy_routed", E, INNER_X, N_EXPERTS), norm, None, norm, None, "l1."))
         return ModelConfig("ToyWindowRouteLM", V, E, NPOS, layers, (LayerCall(0, 0, True), LayerCall(1, 1, True)),
-                           PositionSpec("none"), norm, False, None, (), raw=dict(d))
+                           PositionSpec("none"), norm, False, None, (), raw=dict(d), logit_multiplier=LOGIT_MULT)
 
     def declare(mc):
         q0, q1 = (H0 + 2 * HKV0) * D0, (H1 + 2 * HKV1) * D1
@@ -174,7 +175,7 @@ def plain_toy(W, ids):
         y[rows] = P.gelu_tanh(m[rows] @ W[f"l1.x{e}.fc.weight"].T) @ W[f"l1.x{e}.pr.weight"].T
     x = x + p[:, None] * y
     f = P.layer_norm(x, W["final.weight"], W["final.bias"], EPS)
-    return f @ W["head.weight"].T, np.abs(logits[:, 0] - logits[:, 1])
+    return f @ W["head.weight"].T / LOGIT_MULT, np.abs(logits[:, 0] - logits[:, 1])
 
 
 def test_the_plain_rotation_keeps_what_only_distances_decide():
