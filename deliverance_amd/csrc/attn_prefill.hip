@@ -383,7 +383,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
     // Key phases: a round parks KP tiles (one register set: the next round's loads fly while this
     // round's tiles are multiplied), each wavefront multiplies the tile of its phase.  Two barriers a
     // round: the tiles are parked before anyone reads them and read before they are replaced.
-    fetch(rk0, rv0, kt0);
+    if (b_lo == kt0 && kt0 + KP * PF_BK - 1 <= b_last) fetch_fast(rk0, rv0, kt0);     // (a first round that is whole: no clamping)
+    else fetch(rk0, rv0, kt0);
     for (int kt = kt0; kt <= b_last; kt += KP * PF_BK) {
       stash(rk0, rv0, 0);
       lds_barrier();
