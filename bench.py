@@ -74,8 +74,9 @@ def engine_from_folder(folder, dtype, seats, cfg, **kw):
     from deliverance_amd import AutoModelForCausalLM
     kw.setdefault("max_batch_tokens", max(2048, seats))
     kw.setdefault("max_chunk", 1024)
+    kw.setdefault("page_size", 16)
     return AutoModelForCausalLM.from_pretrained(folder, dtype=dtype, max_num_seqs=max(seats, 2),
-                                                max_cached_tokens=max(seats, 2) * cfg["n_positions"], page_size=16, **kw)
+                                                max_cached_tokens=max(seats, 2) * cfg["n_positions"], **kw)
 
 
 def engine_from_gpu_weights(cfg, dtype, seats, seed=0, **kw):
@@ -105,8 +106,9 @@ def engine_from_gpu_weights(cfg, dtype, seats, seed=0, **kw):
     del tensors
     kw.setdefault("max_batch_tokens", max(2048, seats))
     kw.setdefault("max_chunk", 1024)
+    kw.setdefault("page_size", 16)
     pool = kw.pop("max_cached_tokens", max(seats, 2) * cfg["n_positions"])
-    ec = EngineConfig(dtype=dtype, max_num_seqs=max(seats, 2), max_cached_tokens=pool, page_size=16, **kw)
+    ec = EngineConfig(dtype=dtype, max_num_seqs=max(seats, 2), max_cached_tokens=pool, **kw)
     return CausalLanguageModel(model, ec)
 
 
@@ -230,6 +232,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the GPT-2 1.5B points and the 355M mixed workload")
     ap.add_argument("--profile-stages", action="store_true", help="also print a per-kernel table with roofline fractions (stderr)")
+    ap.add_argument("--page-size", type=int, default=16, choices=[16, 32, 64], help="tokens a cache page")
     ap.add_argument("--prefill-shape", default="2x1024", help="prompts x tokens of the prefill step (the contract's: 2x1024)")
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
@@ -259,7 +262,7 @@ def main():
         return 2
 
     if args.workload == "mixed":
-        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=512 + 64, max_chunk=512,
+        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=512 + 64, max_chunk=512, page_size=args.page_size,
                                         **({"max_cached_tokens": args.pool_tokens} if args.pool_tokens else {}))
         m = mixed_run(model, cfg, rng)
         print(json.dumps({
@@ -269,7 +272,7 @@ def main():
             "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", **{k: m[k] for k in (
                 "seconds", "prompt_tokens", "generated_tokens", "all_tokens_per_second", "requests_equal_in_both_runs")},
             "config": {"model": "gpt2-" + args.model, "n_layer": cfg["n_layer"], "n_embd": cfg["n_embd"],
-                       "n_head": cfg["n_head"], "requests": m["requests"], "max_chunk": 512, "page_size": 16,
+                       "n_head": cfg["n_head"], "requests": m["requests"], "max_chunk": 512, "page_size": args.page_size,
                        "steps": m["steps"], "mean_batch_tokens": m["mean_batch_tokens"], "preemptions": m["preemptions"],
                        "pool_tokens": model.engine_config.max_cached_tokens}}))
         return 0
@@ -277,7 +280,7 @@ def main():
     with tempfile.TemporaryDirectory() as folder:
         random_model(folder, cfg, seed=0)
         model = engine_from_folder(folder, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), cfg,
-                                   kernels=args.kernels, max_batch_tokens=max(2048, args.batch, pf_n * pf_len))
+                                   kernels=args.kernels, max_batch_tokens=max(2048, args.batch, pf_n * pf_len), page_size=args.page_size)
     dt, ctx_mean = decode_run(model, cfg, rng, args.batch, args.prompt_len, args.steps, args.warmup)
     achieved = decode_roofline(cfg, el, args.batch, ctx_mean, dt / args.steps)
     out = {
@@ -289,7 +292,7 @@ def main():
                    "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "n_inner": 4 * cfg["n_embd"],
                    "vocab_size": cfg["vocab_size"], "n_positions": cfg["n_positions"],
                    "global_batch": args.batch, "seq_len": int(round(ctx_mean)),
-                   "prompt_len": args.prompt_len, "page_size": 16, "kernels": args.kernels, "parallelism": "single-gpu"},
+                   "prompt_len": args.prompt_len, "page_size": args.page_size, "kernels": args.kernels, "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
     }
