@@ -50,8 +50,10 @@ __device__ __forceinline__ void kv_scatter_store(const KvScatter& kv, int slot, 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *(const uint4*)p; }
 
 
-// The tiles of 256 x 256 (gemm_wide.hip): what they take, where they pay, and their launch.
+// The tiles whose operands go from memory straight into LDS (gemm_wide.hip): what they take, which of their
+// shapes pays for a product's sizes (DA_WIDE_NONE: none), and their launch.
+enum { DA_WIDE_NONE = -1, DA_WIDE_256x256 = 0, DA_WIDE_256x128 = 1, DA_WIDE_128x128 = 2 };
 bool da_gemm_wide_takes(int act, int accumulate, int out_dtype, int K);
-bool da_gemm_wide_pays(int M, int N);
+extern "C" int da_gemm_wide_choice(int M, int N, int K);
 void da_gemm_wide_launch(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                         const KvScatter& kv, int M, int N, int K);
+                         const KvScatter& kv, int M, int N, int K, int shape);

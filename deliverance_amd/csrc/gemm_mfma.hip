@@ -763,9 +763,10 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     // Smaller tiles where larger ones would leave compute units idle (measured on GPT-2's shapes).
     // Every configuration sums a row's products in the same order (64-wide slabs, 16 at a time), so
     // the choice does not change a result.
-    if (da_gemm_wide_takes(act, accumulate, out_dtype, K) && da_gemm_wide_pays(M, N)) {
-      // tiles of 256 x 256 where they fill the chip: the same sums in the same order, half the LDS traffic
-      da_gemm_wide_launch(s, A, lda, W, ldw, ep, kv, M, N, K);
+    const int wide = da_gemm_wide_takes(act, accumulate, out_dtype, K) ? da_gemm_wide_choice(M, N, K) : DA_WIDE_NONE;
+    if (wide != DA_WIDE_NONE) {
+      // operands straight into LDS where such tiles fill the chip: the same sums in the same order, less LDS traffic
+      da_gemm_wide_launch(s, A, lda, W, ldw, ep, kv, M, N, K, wide);
       DA_CHECK_LAUNCH("gemm_bf16");
       return 0;
     }

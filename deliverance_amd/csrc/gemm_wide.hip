@@ -1,11 +1,14 @@
-// The block-tile product for large steps: tiles of 256 x 256, operands from memory straight into LDS.
+// The block-tile product for large steps: operands from memory straight into LDS.
 //
 //   out[m, n] (+)= act( sum_k a[m, k] * w[n, k] + bias[n] )        (a [M, K], w [N, K], bfloat16, K contiguous)
 //
-// Eight wavefronts, two a SIMD, each with 128 x 64 of the tile (4 x 2 products of 32 x 32 x 16, 128
-// accumulation registers): a k-step of 16 takes 6 fragment reads for 8 matrix instructions, half the LDS
-// traffic a flop of the 128 x 128 tile kernel (gemm_mfma.hip), whose matrix cores wait for LDS most of
-// the time.  A slab of 64 elements of k is 128 bytes a row, one cache line: it goes from memory into LDS
+// The first shape: tiles of 256 x 256, eight wavefronts, two a SIMD, each with 128 x 64 of the tile (4 x 2
+// products of 32 x 32 x 16, 128 accumulation registers): a k-step of 16 takes 6 fragment reads for 8 matrix
+// instructions, half the LDS traffic a flop of the 128 x 128 tile kernel (gemm_mfma.hip), whose matrix cores
+// wait for LDS most of the time.  Two smaller shapes for products whose 256 x 256 tiles would leave compute
+// units idle, their wavefronts with 64 x 64 each (4 reads for 4 matrix instructions): 256 x 128 with eight
+// wavefronts, and 128 x 128 with four, of which two workgroups share a compute unit (da_gemm_wide_choice).
+// A slab of 64 elements of k is 128 bytes a row, one cache line: it goes from memory into LDS
 // without passing registers (da_lds_dma.h), into one of two stages for a (one slab ahead of the
 // products) and one of three for w (two slabs ahead: weights come from memory, not from a cache); one
 // barrier a slab.  Rows lie unpadded in LDS (a copy writes 1,024 consecutive bytes: 8 rows); the
@@ -409,32 +412,49 @@ static void launch_wide(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
   }
 }
 
-// What the wide tiles take: K in whole slabs, and an activation only with a bfloat16 result (the forms
-// that a model's layers use; everything else stays with the 128 x 128 tiles).
+// What these tiles take: K in whole slabs, and an activation only with a bfloat16 result (the forms
+// that a model's layers use; everything else stays with gemm_mfma.hip's tiles).
 bool da_gemm_wide_takes(int act, int accumulate, int out_dtype, int K) {
   return K % WD_BK == 0 && K >= WD_BK && (act == DA_ACT_NONE || (!accumulate && out_dtype == DA_BF16));
 }
 
-// Where they pay: a tile is a compute unit's work for the whole product, so the tiles must fill most of
-// the last round of 256 compute units.  Measured on MI355X with 2,048 rows: ahead of the 128 x 128 tiles
-// from 152 tiles on (N = 4,800: 39 against 47 us; N = 6,400, 200 tiles: 42 against 62 us), behind at 128
-// tiles and fewer (N = 4,096: 30 against 27 us).
-bool da_gemm_wide_pays(int M, int N) {
+// Which shape of tile pays, if any (DA_WIDE_NONE: gemm_mfma.hip's tiles).  A tile is a compute unit's
+// work for the whole product, so the tiles must fill most of the last round of 256 compute units.
+// Measured on MI355X with 256 to 8,192 rows, N from 2,304 to 6,400, K from 768 to 6,400:
+//  - 256 x 256 where its tiles fill 55 % of their last round: ahead of the 128 x 128 tiles from 152 tiles on
+//    (2,048 rows, N = 4,800: 39 against 47 us; N = 6,400, 200 tiles: 42 against 62 us), behind at 128 tiles
+//    and fewer (N = 4,096: 30 against 27 us);
+//  - else, up to a K of 2,048 (beyond, the four slabs in flight of gemm_mfma.hip's tiles win):
+//    256 x 128, one workgroup a compute unit, where 128 x 128 tiles would be 257 to 512, so that some compute
+//    units had two of them and others one (2,048 rows: N = 2,304, K = 768 18.8 against 20.5 us; N = 4,096,
+//    K = 1,024 24.7 against 26.1; 1,536 rows, N = 4,800, K = 1,600 30.6 against 34.7);
+//    128 x 128 of four wavefronts where they are 140 to 256, one a compute unit (1,024 rows, N = 2,304 13.0
+//    against 14.4 us; 512 rows, N = 4,800 19.0 against 23.3; 2,048 rows, N = K = 1,600, += 21.8 against 23.8).
+int da_gemm_wide_choice(int M, int N, int K) {
   const long tiles = (long)da_ceil_div(M, 256) * da_ceil_div(N, 256);
   const long rounds = (tiles + 255) / 256;
-  return tiles * 100 >= rounds * 256 * 55;
+  if (tiles * 100 >= rounds * 256 * 55) return DA_WIDE_256x256;
+  if (K > 2048) return DA_WIDE_NONE;
+  const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
+  if (tiles128 > 256 && tiles128 <= 512) return DA_WIDE_256x128;
+  if (tiles128 >= 140 && tiles128 <= 256) return DA_WIDE_128x128;
+  return DA_WIDE_NONE;
 }
 
 void da_gemm_wide_launch(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                         const KvScatter& kv, int M, int N, int K) {
-  launch_wide<256, 256, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
+                         const KvScatter& kv, int M, int N, int K, int shape) {
+  if (shape == DA_WIDE_128x128) launch_wide<128, 128, 2, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+  else if (shape == DA_WIDE_256x128) launch_wide<256, 128, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+  else launch_wide<256, 256, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
 }
 
-// The wide tiles alone, whatever the shape (tests and timing call it; da_gemm_bf16 chooses by shape).
+// These tiles alone, of the shape asked for (DA_WIDE_256x256, DA_WIDE_256x128, DA_WIDE_128x128), whatever the
+// product's sizes (tests and timing call it; da_gemm_bf16 chooses by them).
 extern "C" int da_gemm_bf16_wide(const void* a, int lda, const void* w, int ldw, const void* bias, int bias_dtype,
                                  int act, int accumulate, void* out, int out_dtype, int ldo, int M, int N, int K,
                                  void* kv_cache, const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
-                                 void* stream) {
+                                 int shape, void* stream) {
+  DA_REQUIRE(shape >= DA_WIDE_256x256 && shape <= DA_WIDE_128x128, "gemm_bf16_wide: unknown tile shape %d", shape);
   DA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16_wide: bad sizes M=%d N=%d K=%d", M, N, K);
   DA_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldo >= N, "gemm_bf16_wide: leading sizes (lda=%d ldw=%d ldo=%d)", lda, ldw, ldo);
   DA_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_wide: operands must be 16-byte aligned");
@@ -448,7 +468,7 @@ extern "C" int da_gemm_bf16_wide(const void* a, int lda, const void* w, int ldw,
   }
   Epilogue ep{bias, bias_dtype, act, accumulate, out, out_dtype, ldo};
   KvScatter kv{kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page};
-  da_gemm_wide_launch((hipStream_t)stream, (const bf16_t*)a, lda, (const bf16_t*)w, ldw, ep, kv, M, N, K);
+  da_gemm_wide_launch((hipStream_t)stream, (const bf16_t*)a, lda, (const bf16_t*)w, ldw, ep, kv, M, N, K, shape);
   DA_CHECK_LAUNCH("gemm_bf16_wide");
   return 0;
 }

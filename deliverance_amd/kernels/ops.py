@@ -76,7 +76,8 @@ _ARGTYPES = {
     "da_layernorm": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _I, _I, _VP],
     "da_gemm_ref": [_VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gemm_bf16": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
-    "da_gemm_bf16_wide": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_bf16_wide": [_VP, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_wide_choice": [_I, _I, _I],
     "da_gemm_bf16_ln": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP,
                         _I, _I, _I, _I, _I, _VP],
     "da_kv_write": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _VP],
@@ -408,13 +409,14 @@ def _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, name):
     return _ptr(kv_cache), _ptr(slot_map), q_cols, Hkv * D, Hkv, D, page
 
 
+WIDE_TILE_SHAPES = {"wide": 0, "wide_256x128": 1, "wide_128x128": 2}
+
+
 def _wide_tiles(M, N, K, act, accumulate, out) -> bool:
-    """Whether the library gives this product to its tiles of 256 x 256 (the profiler's name for it only;
-    the choice itself is the library's: csrc/gemm_wide.hip)."""
-    tiles = -(-M // 256) * -(-N // 256)
-    rounds = -(-tiles // 256)
+    """Whether the library gives this product to its tiles whose operands go straight into LDS (the
+    profiler's name for it only; the choice itself is the library's: csrc/gemm_wide.hip)."""
     takes = K % 64 == 0 and (ACTIVATIONS[act] == 0 or (not accumulate and out.dtype == torch.bfloat16))
-    return takes and tiles * 100 >= rounds * 256 * 55
+    return takes and _lib().da_gemm_wide_choice(M, N, K) >= 0
 
 
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -422,8 +424,9 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
                 slot_map: Optional[torch.Tensor] = None, q_cols: int = 0, form: str = "auto") -> torch.Tensor:
     """out (+)= act(a @ w.T + bias) on the matrix cores; a, w bfloat16, K a multiple of 8.  With
     ``kv_cache`` the columns from ``q_cols`` on (k | v) also go to the cache rows ``slot_map``.
-    ``form``: "auto" lets the library choose by shape; "wide" asks for the tiles of 256 x 256 whose
-    operands go from memory straight into LDS, whatever the shape (K a multiple of 64; tests and timing)."""
+    ``form``: "auto" lets the library choose by shape; "wide", "wide_256x128" and "wide_128x128" ask for the
+    tiles of 256 x 256, 256 x 128 and 128 x 128 whose operands go from memory straight into LDS, whatever
+    the product's sizes (K a multiple of 64; tests and timing)."""
     _dev(a, w, bias, out)
     _rows_2d(a, "a"); _rows_2d(w, "w"); _rows_2d(out, "out")
     M, K = a.shape
@@ -443,13 +446,15 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     if KernelProfiler.enabled:           # (the cost model is worked out only when someone reads it)
         name = "product_skinny" if (M <= 32 or (M <= 64 and N <= 8192)) else ("product_wide" if _wide_tiles(M, N, K, act, accumulate, out) else "product_tile")
         timing = _timed(name, _product_bytes(a, w, bias, out, accumulate), 2 * M * N * K)
-    if form not in ("auto", "wide"):
+    if form != "auto" and form not in WIDE_TILE_SHAPES:
         raise KernelError(f"linear_mfma: unknown form {form!r}")
-    entry = _lib().da_gemm_bf16 if form == "auto" else _lib().da_gemm_bf16_wide
+    args = (_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias), _dt(bias) if bias is not None else 0,
+            ACTIVATIONS[act], int(accumulate), _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp)
     with timing:
-        _check(entry(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias),
-                                   _dt(bias) if bias is not None else 0, ACTIVATIONS[act], int(accumulate),
-                                   _ptr(out), _dt(out), out.stride(0), M, N, K, *kvp, _stream()))
+        if form == "auto":
+            _check(_lib().da_gemm_bf16(*args, _stream()))
+        else:
+            _check(_lib().da_gemm_bf16_wide(*args, WIDE_TILE_SHAPES[form], _stream()))
     return out
 
 

@@ -163,11 +163,13 @@ def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
         assert (out - ref).abs().max() < tol, (act, acc, bias, od)
 
 
+@pytest.mark.parametrize("form", ["wide", "wide_256x128", "wide_128x128"])
 @pytest.mark.parametrize("M,N,K", [helpers.quick(300, 200, 128), (257, 520, 64), (2048, 1600, 320), (700, 4800, 192)])
-def test_gemm_wide_tiles(ops, M, N, K, form="wide"):
-    """The tiles of 256 x 256 whose operands go from memory straight into LDS (two stages of a, three of
-    w): every epilogue against 64-bit arithmetic, and bit for bit what the other tile forms give (all sum
-    over k in ascending steps of 16); edges in M and N, one to five slabs."""
+def test_gemm_wide_tiles(ops, M, N, K, form):
+    """The tiles whose operands go from memory straight into LDS (two stages of a, three of w), in their
+    three shapes (256 x 256, 256 x 128, 128 x 128): every epilogue against 64-bit arithmetic, and bit for
+    bit what the other tile forms give (all sum over k in ascending steps of 16); edges in M and N, one to
+    five slabs."""
     g = torch.Generator().manual_seed(M + N + K)
     wide = lambda *a_, **k_: ops.linear_mfma(*a_, form=form, **k_)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
@@ -189,8 +191,9 @@ def test_gemm_wide_tiles(ops, M, N, K, form="wide"):
         ops.linear_mfma(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous(), b, o1, form=form)
 
 
+@pytest.mark.parametrize("form", ["wide", "wide_256x128", "wide_128x128"])
 @pytest.mark.parametrize("M", [helpers.quick(300), 1000])
-def test_gemm_wide_tiles_write_keys_and_values(ops, M, form="wide"):
+def test_gemm_wide_tiles_write_keys_and_values(ops, M, form):
     g = torch.Generator().manual_seed(M)
     Hq, Hkv, D, page, K = 5, 3, 48, 16, 128
     N = (Hq + 2 * Hkv) * D
