@@ -6,8 +6,8 @@
 // products of 32 x 32 x 16, 128 accumulation registers): a k-step of 16 takes 6 fragment reads for 8 matrix
 // instructions, half the LDS traffic a flop of the 128 x 128 tile kernel (gemm_mfma.hip), whose matrix cores
 // wait for LDS most of the time.  Two smaller shapes for products whose 256 x 256 tiles would leave compute
-// units idle, their wavefronts with 64 x 64 each (4 reads for 4 matrix instructions): 256 x 128 with eight
-// wavefronts, and 128 x 128 with four, of which two workgroups share a compute unit (da_gemm_wide_choice).
+// units idle, both with eight wavefronts: 256 x 128 (64 x 64 a wavefront: 4 reads for 4 matrix instructions),
+// and 128 x 128 (32 x 64 a wavefront), of which two workgroups share a compute unit (da_gemm_wide_choice).
 // A slab of 64 elements of k is 128 bytes a row, one cache line: it goes from memory into LDS
 // without passing registers (da_lds_dma.h), into one of two stages for a (one slab ahead of the
 // products) and one of three for w (two slabs ahead: weights come from memory, not from a cache); one
@@ -353,7 +353,7 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
     // The slab's last k-step, its products one by one, and between them the copies and the reads of slab
     // s + 1's first fragments: the matrix cores have work while the wavefront issues the rest.
     constexpr int CPQ = (CA + CW + TM * TN - 1) / (TM * TN);      // copies after each product
-    static_assert(TM + TN <= TM * TN, "a read for every product at most");
+    constexpr int RPQ = (TM + TN + TM * TN - 1) / (TM * TN);      // reads after each product
 #pragma unroll
     for (int q = 0; q < TM * TN; ++q) {
       WD_MFMA1(fa1, fb1, q);
@@ -362,8 +362,13 @@ gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict
         if (COPY_A && c < CA) WD_COPY_A(c, sa);
         if (COPY_W && c >= CA && c < CA + CW) WD_COPY_W(c - CA, sw);
       }
-      if (NEXT && q < TM) fa0[q] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_a + (sa ^ 1) * A_BYTES + k_off[0] + a_off[q]));
-      if (NEXT && q >= TM && q < TM + TN) fb0[q - TM] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_w + sw1 * W_BYTES + k_off[0] + w_off[q - TM]));
+#pragma unroll
+      for (int r = q * RPQ; r < (q + 1) * RPQ; ++r) {             // (a's fragments, then w's)
+        constexpr int LAST_A = TM - 1, LAST_W = TN - 1;
+        const int ia = r < TM ? r : LAST_A, iw = (r >= TM && r < TM + TN) ? r - TM : LAST_W;    // (indices that exist, whatever r)
+        if (NEXT && r < TM) fa0[ia] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_a + (sa ^ 1) * A_BYTES + k_off[0] + a_off[ia]));
+        if (NEXT && r >= TM && r < TM + TN) fb0[iw] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(smem_w + sw1 * W_BYTES + k_off[0] + w_off[iw]));
+      }
       WD_FENCE();
     }
     sw = sw1;
@@ -420,30 +425,32 @@ bool da_gemm_wide_takes(int act, int accumulate, int out_dtype, int K) {
 
 // Which shape of tile pays, if any (DA_WIDE_NONE: gemm_mfma.hip's tiles).  A tile is a compute unit's
 // work for the whole product, so the tiles must fill most of the last round of 256 compute units.
-// Measured on MI355X with 256 to 8,192 rows, N from 2,304 to 6,400, K from 768 to 6,400:
+// Measured on MI355X with 512 to 8,192 rows, N from 768 to 6,400, K from 768 to 6,400, stores and +=:
 //  - 256 x 256 where its tiles fill 55 % of their last round: ahead of the 128 x 128 tiles from 152 tiles on
 //    (2,048 rows, N = 4,800: 39 against 47 us; N = 6,400, 200 tiles: 42 against 62 us), behind at 128 tiles
 //    and fewer (N = 4,096: 30 against 27 us);
-//  - else, up to a K of 2,048 (beyond, the four slabs in flight of gemm_mfma.hip's tiles win):
-//    256 x 128, one workgroup a compute unit, where 128 x 128 tiles would be 257 to 512, so that some compute
-//    units had two of them and others one (2,048 rows: N = 2,304, K = 768 18.8 against 20.5 us; N = 4,096,
-//    K = 1,024 24.7 against 26.1; 1,536 rows, N = 4,800, K = 1,600 30.6 against 34.7);
-//    128 x 128 of four wavefronts where they are 140 to 256, one a compute unit (1,024 rows, N = 2,304 13.0
-//    against 14.4 us; 512 rows, N = 4,800 19.0 against 23.3; 2,048 rows, N = K = 1,600, += 21.8 against 23.8).
+//  - else, where 128 x 128 tiles would be 257 to 512, so that some compute units had two of gemm_mfma.hip's
+//    and others one: up to a K of 2,048 tiles of 256 x 128, one a compute unit (2,048 rows: N = 2,304,
+//    K = 768 16.2 against 18.9 us; N = 3,072, K = 1,024 20.3 against 23.3; 1,536 rows, N = 4,800, K = 1,600
+//    28.8 against 35.3); beyond, 128 x 128, two a compute unit (4,096 rows, N = 1,600, K = 6,400, += 113
+//    against 130 us; 8,192 rows, N = 768, K = 3,072 58 against 69);
+//  - where they would be 140 to 256, one a compute unit: 128 x 128 up to a K of 4,096 (1,024 rows, N = 2,304
+//    10.6 against 13.5 us; 512 rows, N = 4,800 16.7 against 22.3; 2,048 rows, N = K = 1,600, += 21.1 against
+//    23.3; 4,096 rows, N = 1,024, K = 4,096 48.6 against 56.4); beyond, the four slabs in flight of
+//    gemm_mfma.hip's tiles win (2,048 rows, N = 1,600, K = 6,400: 65 against 79 us).
 int da_gemm_wide_choice(int M, int N, int K) {
   const long tiles = (long)da_ceil_div(M, 256) * da_ceil_div(N, 256);
   const long rounds = (tiles + 255) / 256;
   if (tiles * 100 >= rounds * 256 * 55) return DA_WIDE_256x256;
-  if (K > 2048) return DA_WIDE_NONE;
   const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
-  if (tiles128 > 256 && tiles128 <= 512) return DA_WIDE_256x128;
-  if (tiles128 >= 140 && tiles128 <= 256) return DA_WIDE_128x128;
+  if (tiles128 > 256 && tiles128 <= 512) return K <= 2048 ? DA_WIDE_256x128 : DA_WIDE_128x128;
+  if (tiles128 >= 140 && tiles128 <= 256 && K <= 4096) return DA_WIDE_128x128;
   return DA_WIDE_NONE;
 }
 
 void da_gemm_wide_launch(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
                          const KvScatter& kv, int M, int N, int K, int shape) {
-  if (shape == DA_WIDE_128x128) launch_wide<128, 128, 2, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
+  if (shape == DA_WIDE_128x128) launch_wide<128, 128, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
   else if (shape == DA_WIDE_256x128) launch_wide<256, 128, 4, 2>(s, A, lda, W, ldw, ep, kv, M, N, K);
   else launch_wide<256, 256, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
 }
