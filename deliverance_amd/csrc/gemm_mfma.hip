@@ -7,7 +7,7 @@
 //
 //  * gemm_tile: block tiles of 64x64 to 128x128 (MFMA 32x32x16), operands staged through two LDS
 //    buffers, with the next four slabs already in flight in registers.  For steps with many rows
-//    (prefill).  Products that fill the chip with tiles of 256 x 256 go to gemm_wide.hip instead.
+//    (prefill).  Products whose sizes suit them go to gemm_wide.hip's tiles instead (da_gemm_wide_choice).
 //  * gemm_skinny: for M <= 64 (decode).  A workgroup owns 16 output columns; its wavefronts (4 to 12)
 //    split K, pull their part of a and w from memory in whole cache lines, pass it through LDS into
 //    MFMA 16x16x32 fragments and add their sums through LDS in a fixed order.  Bound by the bytes of w.

@@ -192,12 +192,11 @@ wide_epilogue(floatx16 (&acc)[TM][TN], const float (&bias)[TN], char* region, co
 }
 
 // BM x BN: the tile; WM x WN wavefronts of (BM / WM) x (BN / WN) each.  In use: 256 x 256 with 2 x 4
-// wavefronts of 128 x 64, one workgroup a compute unit (160 KB of LDS).  Measured beside it: four wavefronts
-// of 128 x 128 (a third less LDS traffic; 15 to 25 % slower: one wavefront a SIMD has nobody to fill its
-// waits); tiles of 128 x 128 with 2 x 2 wavefronts of 64 x 64, two workgroups a compute unit (80 KB each):
-// 5 to 15 % ahead of gemm_mfma.hip's tiles when timed alone from 200 tiles on, level or behind inside the
-// model, where a and w both come from memory: a slab of such a tile is half a microsecond of products,
-// and one or two slabs ahead do not cover the way from memory (gemm_mfma.hip keeps four in registers).
+// wavefronts of 128 x 64, one workgroup a compute unit (160 KB of LDS); 256 x 128 with 4 x 2 of 64 x 64
+// (112 KB); 128 x 128 with 4 x 2 of 32 x 64, two workgroups a compute unit (80 KB each); which of them
+// for which sizes: da_gemm_wide_choice.  Measured beside them: 256 x 256 with four wavefronts of 128 x 128
+// (a third less LDS traffic; 15 to 25 % slower: one wavefront a SIMD has nobody to fill its waits);
+// 128 x 128 with 2 x 2 wavefronts of 64 x 64 (7 to 10 % behind the eight wavefronts at a short K).
 template <int BM, int BN, int WM, int WN, int ACT, int OUTMODE>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_wide_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
