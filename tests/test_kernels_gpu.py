@@ -150,10 +150,13 @@ def test_gemm_matrix_cores(ops, M, N, K):
         assert (out - ref).abs().max() < tol, (act, acc, bias, od)
 
 
-@pytest.mark.parametrize("M,N,K", [(1600, 2000, 200), (1555, 1999, 320), (2048, 1600, 1600)])
+@pytest.mark.parametrize("M,N,K", [(1600, 2000, 200), (1555, 1999, 320), (2048, 1600, 1600), (1536, 2304, 768), (2048, 2304, 768),
+                                   (4096, 768, 3072), (2500, 1600, 2112), (2048, 1600, 6400)])
 def test_gemm_tiles_alone_on_their_compute_units(ops, M, N, K):
-    """192 to 256 tiles of 128 x 128: the form with four slabs in flight (a K that a slab cuts, a K of
-    five whole slabs, GPT-2 1.5B's out-proj)."""
+    """The library's own choice where 128 x 128 tiles would be 140 to 512: a K that a slab cuts and a long K with
+    192 to 256 tiles (operands through registers, four slabs in flight: GPT-2 1.5B's proj), whole slabs (operands
+    straight into LDS: 128 x 128 tiles for 208 and 216 tiles, GPT-2 1.5B's out-proj among them, and for 260
+    tiles with a K above 2,048; 256 x 128 for 288 tiles, GPT-2 124M's q|k|v; 128 x 128 for 192 tiles and a K of 3,072)."""
     helpers.skip_in_simulation_if(True)
     g = torch.Generator().manual_seed(M + N + K)
     for act, acc, bias, od in ((None, False, True, torch.bfloat16), ("gelu_new", False, True, torch.bfloat16),
