@@ -234,6 +234,8 @@ def main():
     ap.add_argument("--profile-stages", action="store_true", help="also print a per-kernel table with roofline fractions (stderr)")
     ap.add_argument("--page-size", type=int, default=16, choices=[16, 32, 64], help="tokens a cache page")
     ap.add_argument("--prefill-shape", default="2x1024", help="prompts x tokens of the prefill step (the contract's: 2x1024)")
+    ap.add_argument("--step-tokens", type=int, default=512 + 64,
+                    help="mixed workload: the most tokens a step holds, decoded tokens and a prompt portion together (default: a portion of 512 beside 64 decoded tokens)")
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
                          "requests out of the cache and back, which the line reports as preemptions)")
@@ -262,7 +264,7 @@ def main():
         return 2
 
     if args.workload == "mixed":
-        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=512 + 64, max_chunk=512, page_size=args.page_size,
+        model = engine_from_gpu_weights(cfg, args.dtype, 64, kernels=args.kernels, max_batch_tokens=args.step_tokens, max_chunk=512, page_size=args.page_size,
                                         **({"max_cached_tokens": args.pool_tokens} if args.pool_tokens else {}))
         m = mixed_run(model, cfg, rng)
         print(json.dumps({
@@ -272,7 +274,7 @@ def main():
             "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", **{k: m[k] for k in (
                 "seconds", "prompt_tokens", "generated_tokens", "all_tokens_per_second", "requests_equal_in_both_runs")},
             "config": {"model": "gpt2-" + args.model, "n_layer": cfg["n_layer"], "n_embd": cfg["n_embd"],
-                       "n_head": cfg["n_head"], "requests": m["requests"], "max_chunk": 512, "page_size": args.page_size,
+                       "n_head": cfg["n_head"], "requests": m["requests"], "max_chunk": 512, "step_tokens": args.step_tokens, "page_size": args.page_size,
                        "steps": m["steps"], "mean_batch_tokens": m["mean_batch_tokens"], "preemptions": m["preemptions"],
                        "pool_tokens": model.engine_config.max_cached_tokens}}))
         return 0
